@@ -1,0 +1,229 @@
+#!/usr/bin/env python3
+"""Benchmark of the bitmap SpMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--n N] [--sparsity S]
+
+A step is one SpMM call (main kernel + split-K reduction when the library's
+automatic Split_K is > 1) over one resident compressed copy of the weight
+matrix.  Calls rotate over enough copies of the weights that successive steps
+cannot be served from the 256 MB last-level cache.  Prints one JSON line:
+dense-equivalent TFLOP/s as `value`, plus `roofline` (HBM, algorithmic bytes
+over the main kernel's event-timed duration) and `cpu_baseline` (the CPU
+checker timed on this machine's host cores over a bounded row slice).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+LLC_BYTES = 256 << 20
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--workload", default="opt30b_ffn1")
+    p.add_argument("--n", type=int, default=None, help="override the workload's N")
+    p.add_argument("--sparsity", type=float, default=None, help="override the workload's sparsity (0..1)")
+    p.add_argument("--split-k", type=int, default=0, help="0 = the library's automatic choice")
+    p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--no-dense", action="store_true")
+    p.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    return p.parse_args()
+
+
+class Hip:
+    """The few HIP runtime calls the timing needs (events on the launch stream)."""
+
+    def __init__(self):
+        self.rt = ctypes.CDLL("libamdhip64.so")
+        self.rt.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.rt.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        self.rt.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+        self.rt.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.rt.hipEventDestroy.argtypes = [ctypes.c_void_p]
+
+    def event(self):
+        e = ctypes.c_void_p()
+        assert self.rt.hipEventCreate(ctypes.byref(e)) == 0
+        return e
+
+    def elapsed_ms(self, a, b):
+        ms = ctypes.c_float()
+        assert self.rt.hipEventElapsedTime(ctypes.byref(ms), a, b) == 0
+        return ms.value
+
+
+def cpu_baseline(comp, X, seconds):
+    """Time the CPU checker (decode + fp32-accumulate product, OpenMP) on a bounded slice of 64-row blocks."""
+    from oracle import oracle as O
+    M, K = comp.M, comp.K
+    N = X.shape[0]
+    nkb = K // 64
+
+    def run(row_blocks):
+        g1 = row_blocks * nkb
+        off = comp.offsets[:g1 + 1]
+        t0 = time.perf_counter()
+        O.spmm(comp.values[:int(off[-1])], comp.bitmaps[:g1 * 64], off, X, row_blocks * 64, N, K, 1, False)
+        return time.perf_counter() - t0
+
+    probe = min(M // 64, 16)
+    run(min(probe, 2))  # warm the thread pool
+    t_probe = run(probe)
+    blocks = int(min(M // 64, max(probe, probe * seconds / max(t_probe, 1e-6))))
+    t = run(blocks)
+    rows = blocks * 64
+    flops = 2.0 * rows * N * K
+    # the reference's own CPU path is its single-threaded encoder: time our restatement of it as well
+    enc_rows = min(M, 4096)
+    from spmspm_amd.synthetic import make_weight
+    Wenc = make_weight(enc_rows, K, 0.7, seed=1)
+    t0 = time.perf_counter()
+    O.encode(Wenc, enc_rows, K)
+    t_enc = time.perf_counter() - t0
+    return {
+        "value": flops / t / 1e12, "unit": "TFLOP/s", "cores": O.num_threads(), "kind": "port",
+        "sample": f"rows 0..{rows} of {M} (K={K}, N={N}), {t:.2f} s of host decode+GEMM, OpenMP",
+        "seconds": t,
+        "encoder_melems_per_s_1thread": enc_rows * K / t_enc / 1e6,
+    }
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this build drives one GPU; run with --gpus 1 (the path shards by rows with no "
+              "exchange, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    import spmspm_amd as S
+    from spmspm_amd.synthetic import WORKLOADS, make_activations, make_weight
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    w = dict(WORKLOADS[a.workload])
+    if a.n is not None:
+        w["N"] = a.n
+    if a.sparsity is not None:
+        w["sparsity"] = a.sparsity
+    M, K, N = w["M"], w["K"], w["N"]
+    dev = torch.device("cuda:0")
+
+    t0 = time.perf_counter()
+    W = make_weight(M, K, w["sparsity"], seed=a.seed, pruning=w["pruning"])
+    X = make_activations(K, N, seed=a.seed)
+    t_gen = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    comp = S.InitSparseMatrixA_bitmap(W)
+    t_enc = time.perf_counter() - t0
+
+    algo_bytes = comp.algorithmic_bytes(N)
+    copies = max(2, -(-3 * LLC_BYTES // algo_bytes))
+    layers = [S.SparseLinear(comp, device=dev, split_k=a.split_k) for _ in range(copies)]
+    xs = [torch.from_numpy(X.view(np.int16).copy()).to(dev).view(torch.float16) for _ in range(copies)]
+    outs = [torch.empty((N, M), dtype=torch.float16, device=dev) for _ in range(copies)]
+    split_k = a.split_k if a.split_k > 0 else S.SpMM_SplitK_Auto(M, N, K)
+    ws_bytes = S.SpMM_WorkspaceBytes(M, N, K, a.split_k)
+    for l in layers:
+        l.workspace(N)
+
+    hip = Hip()
+    L = S.library()
+    stream = torch.cuda.current_stream()
+    shandle = stream.cuda_stream
+
+    def step(i, ev=None):
+        j = i % copies
+        if ev is not None:
+            L.SpMM_TimeNextCall(ev[0], ev[1])
+        layers[j](xs[j], out=outs[j], stream=stream)
+
+    for i in range(a.warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    # timed region 1: K steps, wall clock between synchronisations -> value
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    # timed region 2: the same K steps with a HIP event pair around every main-kernel launch -> roofline
+    events = [(hip.event(), hip.event()) for _ in range(a.steps)]
+    for i in range(a.steps):
+        step(i, events[i])
+    torch.cuda.synchronize()
+    kern_ms = np.array([hip.elapsed_ms(e0, e1) for e0, e1 in events])
+    for e0, e1 in events:
+        hip.rt.hipEventDestroy(e0), hip.rt.hipEventDestroy(e1)
+
+    ms_per_step = wall / a.steps * 1e3
+    flops = 2.0 * M * N * K
+    value = flops / (wall / a.steps) / 1e12
+    kern_avg_s = float(kern_ms.mean()) / 1e3
+    achieved = algo_bytes / kern_avg_s / 1e9
+
+    # correctness of what was timed: a row sample against float64
+    rows = np.random.default_rng(1).choice(M, 128, replace=False)
+    got = outs[0].cpu().numpy()[:, rows].astype(np.float64)
+    ref = X.astype(np.float64) @ W[rows].astype(np.float64).T
+    max_abs_frac = float(np.abs(got - ref).max() / np.abs(ref).max())
+    rel_l2 = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+
+    dense = None
+    if not a.no_dense:
+        Wd = [torch.from_numpy(W.view(np.int16)).to(dev).view(torch.float16) for _ in range(max(2, -(-3 * LLC_BYTES // (2 * M * K))))]
+        for i in range(5):
+            torch.matmul(xs[0], Wd[i % len(Wd)].t())
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        reps = max(20, a.steps // 4)
+        for i in range(reps):
+            torch.matmul(xs[0], Wd[i % len(Wd)].t())
+        torch.cuda.synchronize()
+        td = (time.perf_counter() - t0) / reps
+        dense = {"ms": td * 1e3, "tflops": flops / td / 1e12, "gbs": (2.0 * M * K + 2 * K * N + 2 * M * N) / td / 1e9,
+                 "what": "torch.matmul fp16 (hipBLASLt), same run, rotating weight copies"}
+        del Wd
+
+    out = {
+        "metric": "SpMM dense-equiv TFLOP/s", "value": value, "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": f"{a.workload}: W {M}x{K} fp16 N(0,0.02) {w['pruning']}-pruned to "
+                               f"{w['sparsity'] * 100:.0f}% sparsity, X {K}x{N} U(-1,1), seed {a.seed}",
+                   "M": M, "K": K, "N": N, "sparsity": w["sparsity"], "split_k": split_k,
+                   "weight_copies_rotated": copies, "nnz_padded": int(comp.offsets[-1]),
+                   "workspace_bytes": ws_bytes},
+        "gbs_whole_call": algo_bytes / (wall / a.steps) / 1e9,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": algo_bytes, "kernel": "spmm main kernel",
+                     "kernel_avg_us": kern_avg_s * 1e6, "kernel_min_us": float(kern_ms.min()) * 1e3,
+                     "timing": "HIP event pair around each main-kernel launch, same K steps repeated"},
+        "check": {"max_abs_over_max_ref": max_abs_frac, "rel_l2": rel_l2, "rows_sampled": 128},
+        "dense_fp16": dense,
+        "host": {"generate_s": t_gen, "encode_s": t_enc, "encode_threads": os.cpu_count()},
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(comp, X, a.cpu_seconds)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,165 @@
+/*
+ * C ABI of libSpMM_API.so for gfx950 (MI355X): bitmap-compressed (TCA-BME)
+ * unstructured-sparse SpMM,  C[M x N] = W[M x K] (sparse fp16) * X[K x N]
+ * (dense fp16), fp32 accumulation, fp16 output.
+ *
+ * The library keeps the surface of the reference's libSpMM_API.so: a host
+ * encoder and a split-K SpMM entry point.  Each declaration cites the
+ * reference interface it replaces (paths relative to the reference tree).
+ *
+ * Data layouts (identical to the reference's, so encoded weights and
+ * activations are interchangeable):
+ *   W        row-major [M][K] fp16 on the host (encoder input only).
+ *   values   compact non-zero fp16 values, group tile after group tile; each
+ *            64x64 group tile's run is zero-padded to a multiple of 8 halves,
+ *            so every run starts 16-byte aligned.
+ *   bitmaps  one uint64 per 8x8 tile, 64 per group tile; bit r*8+c is element
+ *            (r, c).  Storage index of a tile:
+ *            t = 64*g + 16*strip + 4*q + 2*j + i,  g = gm*(K/64) + gk,
+ *            rows 64*gm + 16*strip + 8*i .. +7, columns 64*gk + 16*q + 8*j .. +7.
+ *   offsets  (TileOffsets_global) G+1 ints, exclusive prefix sum of the padded
+ *            per-group-tile value counts; G = (M/64)*(K/64).
+ *   X        [N][K] fp16 (element (k, n) at X[k + n*K]).
+ *   C        [N][M] fp16 (element (m, n) at C[m + n*M]); fully overwritten.
+ * M and K must be multiples of 64.  N must be 8, 16, 32, 64 or a multiple
+ * of 128.  All SpMM pointer arguments are device memory; calls are
+ * asynchronous on `stream` and never synchronise the host.
+ *
+ * fp16 buffers are typed `void*` / `uint16_t*` so that this header needs no
+ * HIP header; `half*` arguments convert implicitly.
+ */
+#ifndef SPMM_API_H
+#define SPMM_API_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#ifndef HIP_INCLUDE_HIP_HIP_RUNTIME_API_H
+typedef struct ihipStream_t* hipStream_t;
+typedef struct ihipEvent_t*  hipEvent_t;
+#endif
+
+/*
+ * SpMM, north-star form.  Replaces SpMM_SplitK_API_bitmap_v3
+ * (csrc/SpMM_API.cuh:47-110; original 14-argument dense-X form as called at
+ * kernel_benchmark/spmm_test.cu:375-388 and third_party/ft_spinfer.patch:3736-3749)
+ * with the arguments the gfx950 kernel actually needs: strip offsets and the
+ * max-nnz hint are derived from the bitmaps on the device.
+ *
+ *   Split_K >= 1  use that many K batches (partition as in
+ *                 csrc/SpMM_Kernel.cuh:35-43);
+ *   Split_K <= 0  the library picks one for the shape (SpMM_SplitK_Auto).
+ * When the effective Split_K is > 1, `workspace` must hold
+ * SpMM_WorkspaceBytes(M, N, K, Split_K) bytes: partial sums are kept in fp32
+ * (4*M*N*Split_K bytes) and reduced to fp16 by a second kernel.  It may be
+ * NULL when the effective Split_K is 1.
+ * Returns a hipError_t value as int: 0 on success; 999 (hipErrorUnknown) with
+ * the reference's message for an unsupported N (csrc/SpMM_API.cuh:91-94);
+ * 1 (hipErrorInvalidValue) for M or K not a multiple of 64 or a missing
+ * workspace; otherwise the launch status (csrc/SpMM_API.cuh:99-109).
+ */
+int SpMM_SplitK_API(hipStream_t stream, const void* values, const uint64_t* bitmaps, const int* offsets,
+                    const void* X, void* C, int M, int N, int K, void* workspace, int Split_K);
+
+/*
+ * SpMM, reference call-site form: same argument order as the 14-argument
+ * SpMM_SplitK_API_bitmap_v3 the reference's callers use
+ * (kernel_benchmark/spmm_test.cu:375-388, third_party/ft_spinfer.patch:3736-3749),
+ * with hipStream_t for cudaStream_t, so those callers port by type
+ * substitution.  `A` (dense W) is unused and may be NULL, as in the reference.
+ * `TileOffsets` is TileOffsets_global.  `TileOffsets_Median` and
+ * `max_nnz_intile` are accepted for compatibility and not read.
+ * The workspace contract is the reference's: M*N*Split_K halves
+ * (kernel_benchmark/spmm_test.cu:361), partial sums stored as fp16
+ * (csrc/SpMM_Kernel.cuh:192-198) and summed in fp32
+ * (csrc/Reduction_Kernel.cuh:24-45).  Split_K must be >= 1.
+ */
+int SpMM_SplitK_API_bitmap_v3(hipStream_t stream, const void* A, const void* Compressed_A, const int* TileOffsets,
+                              const int* TileOffsets_Median, const uint64_t* bitmap, const int* max_nnz_intile,
+                              const void* B, void* C, int M_Global, int N_Global, int K_Global,
+                              void* Reduction_Workspace, int Split_K);
+
+/*
+ * Split_K the library would pick for a shape when asked to (Split_K <= 0).
+ * Replaces the offline per-matrix table SplitKDict
+ * (end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:23).
+ */
+int SpMM_SplitK_Auto(int M, int N, int K);
+
+/* Bytes of workspace SpMM_SplitK_API needs for this call (0 when the
+ * effective Split_K is 1).  Split_K <= 0 means the automatic choice. */
+size_t SpMM_WorkspaceBytes(int M, int N, int K, int Split_K);
+
+/*
+ * Host encoder, C twin of InitSparseMatrixA_bitmap
+ * (csrc/SpMM_API.cuh:112-241): dense row-major fp16 W -> TCA-BME arrays.
+ * Output is bit-identical to the reference's.  The tile-size arguments are
+ * kept for signature compatibility and must be 8,16,64,8,64,64 (the only
+ * values any reference call site passes); anything else returns -2.
+ * The five output buffers are malloc'd and owned by the caller (free()):
+ *   Compressed_Val      TileOffsets_global[G] halves
+ *   TileOffsets         per-8x8-tile non-zero counts, (M/8)*(K/8) ints
+ *   TileOffsets_median  4*G ints, strip start offsets inside each group tile
+ *   TileOffsets_global  G+1 ints
+ *   bitmap              (M/8)*(K/8) uint64
+ * *max_nnz_count receives the largest padded per-group-tile count (callers
+ * round it up to a multiple of 64, csrc/SpMM_API.cuh:284-286).
+ * Returns G = (M/64)*(K/64), or -1 if an allocation fails (:141-144).
+ * Rows/columns beyond the last multiple of 64 are ignored, as in the
+ * reference (:130-132).
+ */
+int InitSparseMatrixA_bitmap(uint16_t* A_h, int M, int K, int tile_M, int tile_M_median, int tile_M_global,
+                             int tile_K, int tile_K_median, int tile_K_global, uint16_t** Compressed_Val,
+                             int** TileOffsets, int** TileOffsets_median, int** TileOffsets_global,
+                             uint64_t** bitmap, int* max_nnz_count);
+
+/*
+ * File-to-file encoder, replaces Our_GenSparseMatrixBinFile
+ * (csrc/SpMM_API.cuh:243-320; called through ctypes at
+ * end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:88-102).
+ * Reads M*K fp16 from DenseMatrixFileName and writes the six files the
+ * reference writes, byte for byte: values, TileOffsets_global (G+1 ints),
+ * TileOffsets_median (4G ints), bitmaps (64G uint64), max_nnz rounded up to a
+ * multiple of 64 (1 int), and sizes {val_count, G+1, 4G, 64G} (4 ints).
+ * Like the reference it prints a message and exits the process with -1 when a
+ * file cannot be opened or is too short.
+ */
+void Our_GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int K, char* Compressed_ValFileName,
+                                char* bitmap_TileOffsets_globalFileName, char* bitmap_TileOffsets_medianFileName,
+                                char* bitmapFileName, char* max_nnz_intileFileName, char* OutputSizesFileName);
+
+/*
+ * Timing aid with no counterpart in the reference (its harness times whole
+ * calls with cudaEvents, kernel_benchmark/spmm_test.cu:374-411): the next SpMM
+ * call made by this thread records `before_main` on its stream just before it
+ * launches the main kernel and `after_main` just after, so a caller can read
+ * the main kernel's duration apart from the split-K reduction.  Either may be
+ * NULL.  The request is consumed by that one call.
+ */
+void SpMM_TimeNextCall(hipEvent_t before_main, hipEvent_t after_main);
+
+/* Library version string, e.g. "spmm-gfx950 0.1". */
+const char* SpMM_Version(void);
+
+#ifdef __cplusplus
+} /* extern "C" */
+
+#if defined(HIP_INCLUDE_HIP_HIP_FP16_H) || defined(SPMM_API_WITH_HALF)
+/*
+ * C++ overload with the reference's exact signature and mangled name
+ * (_Z24InitSparseMatrixA_bitmapP6__halfiiiiiiiiPS0_PPiS3_S3_PPmRi,
+ * csrc/SpMM_API.cuh:112-120), for callers compiled against the reference.
+ * Declared when <hip/hip_fp16.h> was included first.
+ */
+int InitSparseMatrixA_bitmap(__half* A_h, int M, int K, int tile_M, int tile_M_median, int tile_M_global, int tile_K,
+                             int tile_K_median, int tile_K_global, __half** Compressed_Val, int** TileOffsets,
+                             int** TileOffsets_median, int** TileOffsets_global, uint64_t** bitmap,
+                             int& max_nnz_count);
+#endif
+#endif /* __cplusplus */
+
+#endif /* SPMM_API_H */

@@ -1,0 +1,19 @@
+"""MI355X (gfx950) bitmap-compressed SpMM: host layer over libSpMM_API.so.
+
+The functions mirror the reference's public interface for this path
+(csrc/SpMM_API.cuh): `InitSparseMatrixA_bitmap` (host encoder) and
+`SpMM_SplitK_API` / `SpMM_SplitK_API_bitmap_v3` (device SpMM).
+"""
+from .api import (  # noqa: F401
+    CompressedMatrix,
+    InitSparseMatrixA_bitmap,
+    Our_GenSparseMatrixBinFile,
+    SparseLinear,
+    SpMM_SplitK_API,
+    SpMM_SplitK_API_bitmap_v3,
+    SpMM_SplitK_Auto,
+    SpMM_WorkspaceBytes,
+    library,
+    library_path,
+    load_weight_files,
+)

@@ -1,0 +1,48 @@
+"""Builds libSpMM_API.so for gfx950 in-tree (spmspm_amd/lib/)."""
+import os
+import shutil
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+LIBDIR = os.path.join(PKG, "lib")
+LIBPATH = os.path.join(LIBDIR, "libSpMM_API.so")
+
+SOURCES = ["spmm_api.hip", "encoder.cpp"]
+# Packed-fp32 VALU forms are switched off for every device compile.
+HIPCC_FLAGS = [
+    "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared", "-fvisibility=default",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
+]
+
+
+def hipcc():
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; the ROCm toolchain is required to build libSpMM_API.so")
+    return exe
+
+
+def build_library(verbose=False, extra_flags=()):
+    """Compile every source into one shared library.  Always recompiles."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    cmd = [hipcc(), *HIPCC_FLAGS, *extra_flags, "-I", os.path.join(ROOT, "include"), "-I", CSRC]
+    cmd += [os.path.join(CSRC, s) for s in SOURCES]
+    cmd += ["-o", LIBPATH + ".tmp", "-lpthread"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        sys.stderr.write(proc.stdout + proc.stderr)
+        raise RuntimeError("hipcc failed building libSpMM_API.so")
+    if verbose and proc.stderr.strip():
+        sys.stderr.write(proc.stderr)
+    os.replace(LIBPATH + ".tmp", LIBPATH)
+    return LIBPATH
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

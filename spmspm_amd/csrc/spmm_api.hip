@@ -1,0 +1,149 @@
+// Dispatcher, launcher and C ABI of the gfx950 bitmap SpMM.
+// Replaces the host side of csrc/SpMM_API.cuh:21-110.
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdio>
+#include <cstdlib>
+
+#include "spmm_api.h"
+#include "spmm_kernels.hiph"
+
+namespace {
+
+bool supported_n(int N)
+{
+    // The reference's switch (csrc/SpMM_API.cuh:60-96).
+    return N == 8 || N == 16 || N == 32 || N == 64 || (N > 0 && N % 128 == 0);
+}
+
+int clamp_split_k(int split_k, int K)
+{
+    const int nkb = K / 64;
+    if (split_k > nkb)
+        split_k = nkb; // more batches than group-tile columns would leave empty batches
+    return split_k < 1 ? 1 : split_k;
+}
+
+// Work-fill heuristic: enough workgroups that every one of the 256 CUs holds a
+// few, while each batch still walks a useful number of group tiles.
+int auto_split_k(int M, int N, int K)
+{
+    const int  nkb        = K / 64;
+    const int  row_blocks = M / 64;
+    const int  col_blocks = spmm::column_blocks(N);
+    const long target     = 256L * 4;
+    long       base       = (long)row_blocks * col_blocks;
+    if (base <= 0 || nkb <= 0)
+        return 1;
+    int sk = (int)((target + base - 1) / base);
+    // keep at least 8 group tiles per batch (2 per wave) unless K itself is shorter
+    int max_sk = nkb / 8;
+    if (max_sk < 1)
+        max_sk = 1;
+    if (sk > max_sk)
+        sk = max_sk;
+    if (sk < 1)
+        sk = 1;
+    return sk;
+}
+
+int check_shape(int M, int N, int K)
+{
+    if (!supported_n(N)) {
+        std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", N);
+        std::fflush(stdout);
+        return (int)hipErrorUnknown;
+    }
+    if (M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0) {
+        std::printf("MM_Sparse_API Error: M (%d) and K (%d) must be positive multiples of 64!\n", M, K);
+        std::fflush(stdout);
+        return (int)hipErrorInvalidValue;
+    }
+    return 0;
+}
+
+// Optional timing hooks: the next SpMM call on this thread records these around its main kernel.
+thread_local hipEvent_t t_before_main = nullptr;
+thread_local hipEvent_t t_after_main  = nullptr;
+
+int run(hipStream_t stream, const void* values, const uint64_t* bitmaps, const int* offsets, const void* X, void* C,
+        int M, int N, int K, void* workspace, int split_k, bool fp32_partials)
+{
+    if (int e = check_shape(M, N, K))
+        return e;
+    split_k = clamp_split_k(split_k, K);
+    if (split_k > 1 && workspace == nullptr) {
+        std::printf("MM_Sparse_API Error: Split_K=%d needs a reduction workspace!\n", split_k);
+        std::fflush(stdout);
+        return (int)hipErrorInvalidValue;
+    }
+    (void)hipGetLastError(); // do not report a stale error as ours
+    hipEvent_t before = t_before_main, after = t_after_main;
+    t_before_main = t_after_main = nullptr;
+    if (before)
+        (void)hipEventRecord(before, stream);
+    spmm::launch_spmm(stream, static_cast<const __half*>(values), bitmaps, offsets, static_cast<const __half*>(X),
+                      static_cast<__half*>(C), M, N, K, workspace, split_k, fp32_partials);
+    if (after)
+        (void)hipEventRecord(after, stream);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess || split_k == 1)
+        return (int)err;
+    spmm::launch_reduction(stream, static_cast<__half*>(C), workspace, M, N, split_k, fp32_partials);
+    return (int)hipGetLastError();
+}
+
+} // namespace
+
+extern "C" int SpMM_SplitK_Auto(int M, int N, int K)
+{
+    if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
+        return 1;
+    return clamp_split_k(auto_split_k(M, N, K), K);
+}
+
+extern "C" size_t SpMM_WorkspaceBytes(int M, int N, int K, int Split_K)
+{
+    int sk = Split_K <= 0 ? SpMM_SplitK_Auto(M, N, K) : clamp_split_k(Split_K, K);
+    if (sk <= 1)
+        return 0;
+    return sizeof(float) * (size_t)M * (size_t)N * (size_t)sk;
+}
+
+extern "C" int SpMM_SplitK_API(hipStream_t stream, const void* values, const uint64_t* bitmaps, const int* offsets,
+                               const void* X, void* C, int M, int N, int K, void* workspace, int Split_K)
+{
+    if (int e = check_shape(M, N, K))
+        return e;
+    int sk = Split_K <= 0 ? SpMM_SplitK_Auto(M, N, K) : Split_K;
+    return run(stream, values, bitmaps, offsets, X, C, M, N, K, workspace, sk, /*fp32_partials=*/true);
+}
+
+extern "C" int SpMM_SplitK_API_bitmap_v3(hipStream_t stream, const void* /*A*/, const void* Compressed_A,
+                                         const int* TileOffsets, const int* /*TileOffsets_Median*/,
+                                         const uint64_t* bitmap, const int* /*max_nnz_intile*/, const void* B,
+                                         void* C, int M_Global, int N_Global, int K_Global,
+                                         void* Reduction_Workspace, int Split_K)
+{
+    if (int e = check_shape(M_Global, N_Global, K_Global))
+        return e;
+    if (Split_K < 1) {
+        std::printf("MM_Sparse_API Error: Split_K (%d) must be >= 1!\n", Split_K);
+        std::fflush(stdout);
+        return (int)hipErrorInvalidValue;
+    }
+    return run(stream, Compressed_A, bitmap, TileOffsets, B, C, M_Global, N_Global, K_Global, Reduction_Workspace,
+               Split_K, /*fp32_partials=*/false);
+}
+
+extern "C" void SpMM_TimeNextCall(hipEvent_t before_main, hipEvent_t after_main)
+{
+    t_before_main = before_main;
+    t_after_main  = after_main;
+}
+
+extern "C" const char* SpMM_Version(void)
+{
+    return "spmm-gfx950 0.1";
+}

@@ -1,0 +1,244 @@
+"""Parity of the HIP SpMM (through the C ABI) with the CPU oracle, the golden vectors and float64 mathematics."""
+import numpy as np
+import pytest
+
+import spmspm_amd as S
+from conftest import assert_spmm_close
+from spmspm_amd.synthetic import make_activations, make_weight
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+class Device:
+    """Uploads one compressed matrix the way the reference's harness does (kernel_benchmark/spmm_test.cu:334-372)."""
+
+    def __init__(self, torch, comp):
+        self.torch = torch
+        self.c = comp
+        dev = "cuda:0"
+        vals = comp.values if comp.values.size else np.zeros(8, np.uint16)
+        self.values = torch.from_numpy(vals.view(np.int16).copy()).to(dev)
+        self.bitmaps = torch.from_numpy(comp.bitmaps.view(np.int64).copy()).to(dev)
+        self.offsets = torch.from_numpy(comp.offsets.copy()).to(dev)
+        self.median = torch.from_numpy(comp.median.copy() if comp.median.size else np.zeros(4, np.int32)).to(dev)
+        self.max_nnz = torch.tensor([comp.max_nnz_rounded], dtype=torch.int32, device=dev)
+
+    def spmm(self, X, split_k, entry="api"):
+        torch = self.torch
+        N, K = X.shape
+        M = self.c.M
+        x = torch.from_numpy(X.view(np.int16).copy()).to("cuda:0")
+        out = torch.full((N, M), 0x7e00, dtype=torch.int16, device="cuda:0")  # NaN-filled: C must be overwritten
+        if entry == "api":
+            nbytes = S.SpMM_WorkspaceBytes(M, N, K, split_k)
+            ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda:0") if nbytes else None
+            err = S.SpMM_SplitK_API(None, self.values, self.bitmaps, self.offsets, x, out, M, N, K, ws, split_k)
+        else:
+            ws = torch.empty(max(2 * M * N * max(split_k, 1), 16), dtype=torch.uint8, device="cuda:0")
+            err = S.SpMM_SplitK_API_bitmap_v3(None, None, self.values, self.offsets, self.median, self.bitmaps,
+                                              self.max_nnz, x, out, M, N, K, ws, split_k)
+        assert err == 0, f"hipError_t {err}"
+        torch.cuda.synchronize()
+        return out.cpu().numpy().view(np.float16)
+
+
+def _oracle_C(oracle, comp, X, split_k=1, partial_fp16=False):
+    N, K = X.shape
+    return oracle.spmm(comp.values, comp.bitmaps, comp.offsets, X, comp.M, N, K, split_k, partial_fp16)
+
+
+SHAPES = [
+    # M, K, N, sparsity, split_k
+    (64, 64, 16, 0.5, 1),
+    (64, 64, 8, 0.5, 1),
+    (128, 192, 16, 0.7, 1),
+    (256, 256, 32, 0.5, 1),
+    (256, 512, 64, 0.6, 1),
+    (128, 256, 128, 0.4, 1),
+    (64, 128, 256, 0.5, 1),
+    (256, 1024, 16, 0.7, 3),
+    (256, 1024, 16, 0.7, 4),
+    (192, 576, 8, 0.6, 2),
+    (128, 640, 32, 0.5, 5),
+    (128, 512, 64, 0.5, 7),
+    (64, 320, 128, 0.5, 5),
+    (512, 2048, 16, 0.9, 8),
+    (1024, 1024, 16, 0.0, 2),
+    (256, 256, 16, 1.0, 2),
+]
+
+
+@pytest.mark.parametrize("M,K,N,s,sk", SHAPES)
+def test_matches_oracle(torch, oracle, M, K, N, s, sk):
+    W = make_weight(M, K, s, seed=M + K + N)
+    X = make_activations(K, N, seed=N)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    dev = Device(torch, comp)
+    print(f"case M={M} K={K} N={N} s={s} sk={sk}", flush=True)
+    C = dev.spmm(X, sk, "api")
+    ref64 = X.astype(np.float64) @ W.astype(np.float64).T
+    assert_spmm_close(C, _oracle_C(oracle, comp, X, sk, False), "api vs oracle")
+    assert_spmm_close(C, ref64, "api vs float64")
+    Cv3 = dev.spmm(X, sk, "v3")
+    assert_spmm_close(Cv3, _oracle_C(oracle, comp, X, sk, True), "v3 vs oracle (fp16 partials)")
+    assert_spmm_close(Cv3, ref64, "v3 vs float64")
+
+
+def test_exact_on_small_integers(torch, oracle):
+    """Where fp32 accumulation is exact the result must be bit-identical to the oracle, any Split_K."""
+    rng = np.random.default_rng(5)
+    M, K, N = 256, 512, 16
+    W = rng.integers(-3, 4, (M, K)).astype(np.float16)
+    W[rng.random((M, K)) < 0.6] = 0
+    X = rng.integers(-2, 3, (N, K)).astype(np.float16)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    dev = Device(torch, comp)
+    want = _oracle_C(oracle, comp, X).view(np.uint16)
+    for sk in (1, 2, 4, 8):
+        for entry in ("api", "v3"):
+            got = dev.spmm(X, sk, entry).view(np.uint16)
+            assert np.array_equal(got, want), (sk, entry)
+
+
+def test_golden_fixtures_decode_on_device(torch, golden):
+    """Every committed golden encoding multiplies to the same product as its dense input."""
+    for name, g in golden.items():
+        M, K = g["W"].shape
+        Mt, Kt = M // 64 * 64, K // 64 * 64
+        if Mt == 0 or Kt == 0:
+            continue
+        comp = S.CompressedMatrix(M=Mt, K=Kt, num_gtiles=int(g["scalars"][0]), values=g["values"],
+                                  tile_counts=g["tile_counts"], median=g["median"], offsets=g["offsets"],
+                                  bitmaps=g["bitmaps"], max_nnz=int(g["scalars"][1]))
+        W = g["W"].view(np.float16)[:Mt, :Kt].astype(np.float64)
+        if not np.isfinite(W).all():
+            continue  # the special-values case is covered by test_special_values_propagate
+        X = make_activations(Kt, 16, seed=1)
+        C = Device(torch, comp).spmm(X, 1)
+        assert_spmm_close(C, X.astype(np.float64) @ W.T, name)
+
+
+def test_special_values_propagate(torch):
+    """-0.0 is dropped by the encoder, NaN/inf/subnormal weights are kept and reach the right outputs."""
+    M, K, N = 64, 128, 16
+    W = np.zeros((M, K), np.float16)
+    W[3, 5] = np.float16(np.nan)
+    W[10, 70] = np.float16(np.inf)
+    W[20, 9] = np.float16(6e-8)  # subnormal
+    W[21, 9] = np.float16(-0.0)
+    W[40, 127] = np.float16(2.0)
+    X = np.ones((N, K), np.float16)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    C = Device(torch, comp).spmm(X, 1)
+    assert np.isnan(C[:, 3]).all() and np.isposinf(C[:, 10]).all()
+    assert (C[:, 20] == np.float16(6e-8)).all() and (C[:, 40] == 2).all()
+    rest = np.delete(C, [3, 10, 20, 40], axis=1)
+    assert not rest.any()
+
+
+def test_ragged_row_populations(torch, oracle):
+    """Group tiles from empty to completely full inside one matrix, every strip offset exercised."""
+    rng = np.random.default_rng(23)
+    M, K, N = 256, 1024, 16
+    W = (rng.standard_normal((M, K)) * 0.02).astype(np.float16)
+    dens = rng.random((M // 64, K // 64))
+    dens[0, 0], dens[1, 3], dens[2, 5] = 0.0, 1.0, 1.0
+    for gm in range(M // 64):
+        for gk in range(K // 64):
+            blk = W[gm * 64:(gm + 1) * 64, gk * 64:(gk + 1) * 64]
+            blk[rng.random((64, 64)) >= dens[gm, gk]] = 0
+    W[64:128, 192:256] = np.where(W[64:128, 192:256] == 0, np.float16(0.01), W[64:128, 192:256])  # truly dense
+    X = make_activations(K, N, seed=2)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    assert comp.max_nnz == 4096
+    dev = Device(torch, comp)
+    for sk in (1, 3):
+        assert_spmm_close(dev.spmm(X, sk), _oracle_C(oracle, comp, X, sk), f"ragged sk={sk}")
+
+
+def test_reference_harness_inputs_and_error_metric(torch, oracle):
+    """The reference's own generator and its sum-of-abs-diff check (kernel_benchmark/spmm_test_utils.h:88-110)."""
+    M = K = 512
+    N = 16
+    W, X = oracle.init_host_matrices(M, K, N, 50, reseed=True)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    C = Device(torch, comp).spmm(X, 1, "v3")
+    ref = (X.astype(np.float64) @ W.astype(np.float64).T)
+    ref16 = ref.astype(np.float16)
+    assert_spmm_close(C, ref, "harness inputs")
+    # values are multiples of 0.1-ish fp16 numbers: total error stays tiny relative to sum|C|
+    assert oracle.total_error(ref16, C) <= 1e-3 * np.abs(ref).sum()
+
+
+def test_auto_split_k_and_invariance(torch, oracle):
+    M, K, N = 512, 4096, 16
+    W = make_weight(M, K, 0.6, seed=4, pruning="magnitude")
+    X = make_activations(K, N, seed=4)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    dev = Device(torch, comp)
+    ref = X.astype(np.float64) @ W.astype(np.float64).T
+    auto = S.SpMM_SplitK_Auto(M, N, K)
+    assert auto > 1
+    for sk in (0, 1, 2, 64, 1000):  # 0 = automatic; 1000 is clamped to K/64
+        assert_spmm_close(dev.spmm(X, sk), ref, f"sk={sk}")
+
+
+def test_linearity_at_full_size(torch):
+    """OPT-13B QKV shape: C(X1 + X2) == C(X1) + C(X2) within the contract, and C(0) == 0."""
+    M, K, N = 15360, 5120, 16
+    W = make_weight(M, K, 0.6, seed=0, pruning="magnitude")
+    comp = S.InitSparseMatrixA_bitmap(W)
+    dev = Device(torch, comp)
+    rng = np.random.default_rng(1)
+    X1 = (rng.integers(-4, 5, (N, K)) / 8).astype(np.float16)
+    X2 = (rng.integers(-4, 5, (N, K)) / 8).astype(np.float16)
+    C1, C2, C12 = dev.spmm(X1, 0), dev.spmm(X2, 0), dev.spmm(X1 + X2, 0)
+    assert_spmm_close(C12, C1.astype(np.float64) + C2.astype(np.float64), "linearity")
+    assert not dev.spmm(np.zeros((N, K), np.float16), 0).any()
+    # a sampled set of rows against float64
+    rows = rng.choice(M, 64, replace=False)
+    ref = X1.astype(np.float64) @ W[rows].astype(np.float64).T
+    assert_spmm_close(C1[:, rows], ref, "sampled rows")
+
+
+def test_target_shape_against_oracle(torch, oracle):
+    """OPT-30B FFN1 28672x7168, 70 % sparse, N=16: whole output against the oracle."""
+    M, K, N = 28672, 7168, 16
+    W = make_weight(M, K, 0.7, seed=0)
+    X = make_activations(K, N, seed=0)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    dev = Device(torch, comp)
+    want = _oracle_C(oracle, comp, X)
+    for sk in (0, 1):
+        assert_spmm_close(dev.spmm(X, sk), want, f"target sk={sk}")
+    assert_spmm_close(dev.spmm(X, 4, "v3"), want, "target v3 sk=4")
+
+
+def test_error_returns_on_device(torch, capfd):
+    t = torch.zeros(16, dtype=torch.int16, device="cuda:0")
+    assert S.SpMM_SplitK_API(None, t, t, t, t, t, 64, 48, 64, None, 1) == S.api.HIP_ERROR_UNKNOWN
+    assert "Unsupported N dimension 48" in capfd.readouterr().out
+    assert S.SpMM_SplitK_API_bitmap_v3(None, None, t, t, t, t, t, t, t, 64, 16, 96, t, 1) == S.api.HIP_ERROR_INVALID_VALUE
+    torch.cuda.synchronize()
+
+
+def test_stream_argument_is_honoured(torch, oracle):
+    M, K, N = 256, 512, 16
+    W = make_weight(M, K, 0.5, seed=8)
+    X = make_activations(K, N, seed=8)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    lin = S.SparseLinear(comp, split_k=2)
+    x = torch.from_numpy(X.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        y = lin(x, stream=side)
+    side.synchronize()
+    assert_spmm_close(y.cpu().numpy(), _oracle_C(oracle, comp, X, 2), "side stream")
