@@ -83,7 +83,12 @@ def cpu_baseline(comp, X, seconds):
     run(min(probe, 2))  # warm the thread pool
     t_probe = run(probe)
     blocks = int(min(M // 64, max(probe, probe * seconds / max(t_probe, 1e-6))))
-    t = run(blocks)
+    t_once = run(blocks)
+    reps = max(1, int(seconds / max(t_once, 1e-6)))  # whole passes over the slice until the time target is met
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        run(blocks)
+    t = (time.perf_counter() - t0) / reps
     rows = blocks * 64
     flops = 2.0 * rows * N * K
     # the reference's own CPU path is its single-threaded encoder: time our restatement of it as well
@@ -95,8 +100,8 @@ def cpu_baseline(comp, X, seconds):
     t_enc = time.perf_counter() - t0
     return {
         "value": flops / t / 1e12, "unit": "TFLOP/s", "cores": O.num_threads(), "kind": "port",
-        "sample": f"rows 0..{rows} of {M} (K={K}, N={N}), {t:.2f} s of host decode+GEMM, OpenMP",
-        "seconds": t,
+        "sample": f"rows 0..{rows} of {M} (K={K}, N={N}), {reps} passes of {t:.3f} s, host decode+GEMM, OpenMP",
+        "seconds_per_pass": t, "passes": reps,
         "encoder_melems_per_s_1thread": enc_rows * K / t_enc / 1e6,
     }
 
