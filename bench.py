@@ -168,7 +168,7 @@ def main():
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
 
-    # timed region 2: the same K steps with a HIP event pair around every main-kernel launch -> roofline
+    # timed region 2: the same K steps with a HIP event pair attached to every main-kernel dispatch -> roofline
     events = [(hip.event(), hip.event()) for _ in range(a.steps)]
     for i in range(a.steps):
         step(i, events[i])
@@ -220,7 +220,8 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": algo_bytes, "kernel": "spmm main kernel",
                      "kernel_avg_us": kern_avg_s * 1e6, "kernel_min_us": float(kern_ms.min()) * 1e3,
-                     "timing": "HIP event pair around each main-kernel launch, same K steps repeated"},
+                     "timing": "HIP events attached to each main-kernel dispatch (kernel begin/end timestamps), "
+                               "same K steps repeated after the wall-clock region"},
         "check": {"max_abs_over_max_ref": max_abs_frac, "rel_l2": rel_l2, "rows_sampled": 128},
         "dense_fp16": dense,
         "host": {"generate_s": t_gen, "encode_s": t_enc, "encode_threads": os.cpu_count()},

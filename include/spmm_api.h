@@ -135,10 +135,11 @@ void Our_GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int K, char* C
 /*
  * Timing aid with no counterpart in the reference (its harness times whole
  * calls with cudaEvents, kernel_benchmark/spmm_test.cu:374-411): the next SpMM
- * call made by this thread records `before_main` on its stream just before it
- * launches the main kernel and `after_main` just after, so a caller can read
- * the main kernel's duration apart from the split-K reduction.  Either may be
- * NULL.  The request is consumed by that one call.
+ * call made by this thread attaches the two events to the dispatch of its main
+ * kernel, so that `before_main` carries the kernel's begin timestamp and
+ * `after_main` its end timestamp; hipEventElapsedTime between them is the main
+ * kernel's duration alone (no launch latency, no split-K reduction).  Either
+ * may be NULL.  The request is consumed by that one call.
  */
 void SpMM_TimeNextCall(hipEvent_t before_main, hipEvent_t after_main);
 

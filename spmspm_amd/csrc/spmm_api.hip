@@ -25,27 +25,38 @@ int clamp_split_k(int split_k, int K)
     return split_k < 1 ? 1 : split_k;
 }
 
-// Work-fill heuristic: enough workgroups that every one of the 256 CUs holds a
-// few, while each batch still walks a useful number of group tiles.
+// Picks the K split from a small cost model (units: group tiles processed by the busiest CU).
+//   work     ceil(workgroups / 256) turns of (tiles per workgroup + a fixed start-up/epilogue cost);
+//   fill     with fewer than four workgroups per CU the waves cannot hide memory latency;
+//   partials every extra batch writes and re-reads an fp32 slab of M*N.
 int auto_split_k(int M, int N, int K)
 {
-    const int  nkb        = K / 64;
-    const int  row_blocks = M / 64;
-    const int  col_blocks = spmm::column_blocks(N);
-    const long target     = 256L * 4;
-    long       base       = (long)row_blocks * col_blocks;
+    const int    nkb  = K / 64;
+    const long   base = (long)(M / 64) * spmm::column_blocks(N);
+    const double kCUs = 256.0, kStartupTiles = 3.0, kTileBytes = 3000.0;
     if (base <= 0 || nkb <= 0)
         return 1;
-    int sk = (int)((target + base - 1) / base);
-    // keep at least 8 group tiles per batch (2 per wave) unless K itself is shorter
-    int max_sk = nkb / 8;
-    if (max_sk < 1)
-        max_sk = 1;
-    if (sk > max_sk)
-        sk = max_sk;
-    if (sk < 1)
-        sk = 1;
-    return sk;
+    int    best    = 1;
+    double best_c  = 1e30;
+    int    max_sk  = nkb / 4 > 0 ? nkb / 4 : 1; // at least one group tile per wave and batch
+    if (max_sk > 32)
+        max_sk = 32;
+    for (int sk = 1; sk <= max_sk; ++sk) {
+        const double wgs   = (double)base * sk;
+        const double turns = (double)((long)((wgs + kCUs - 1) / kCUs));
+        const double tiles = (double)((nkb + sk - 1) / sk) + kStartupTiles;
+        double       cost  = turns * tiles;
+        const double per_cu = wgs / kCUs;
+        if (per_cu < 4.0)
+            cost *= 4.0 / (per_cu < 0.25 ? 0.25 : per_cu);
+        if (sk > 1)
+            cost += sk * ((double)M * N * 8.0 / kCUs) / kTileBytes;
+        if (cost < best_c - 1e-9) {
+            best_c = cost;
+            best   = sk;
+        }
+    }
+    return best;
 }
 
 int check_shape(int M, int N, int K)
@@ -63,7 +74,7 @@ int check_shape(int M, int N, int K)
     return 0;
 }
 
-// Optional timing hooks: the next SpMM call on this thread records these around its main kernel.
+// Optional timing hooks: the next SpMM call on this thread attaches these to its main kernel's dispatch.
 thread_local hipEvent_t t_before_main = nullptr;
 thread_local hipEvent_t t_after_main  = nullptr;
 
@@ -81,12 +92,8 @@ int run(hipStream_t stream, const void* values, const uint64_t* bitmaps, const i
     (void)hipGetLastError(); // do not report a stale error as ours
     hipEvent_t before = t_before_main, after = t_after_main;
     t_before_main = t_after_main = nullptr;
-    if (before)
-        (void)hipEventRecord(before, stream);
     spmm::launch_spmm(stream, static_cast<const __half*>(values), bitmaps, offsets, static_cast<const __half*>(X),
-                      static_cast<__half*>(C), M, N, K, workspace, split_k, fp32_partials);
-    if (after)
-        (void)hipEventRecord(after, stream);
+                      static_cast<__half*>(C), M, N, K, workspace, split_k, fp32_partials, before, after);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess || split_k == 1)
         return (int)err;
