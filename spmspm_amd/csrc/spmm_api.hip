@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 
@@ -112,7 +113,11 @@ extern "C" int SpMM_SplitK_Auto(int M, int N, int K)
 
 extern "C" size_t SpMM_WorkspaceBytes(int M, int N, int K, int Split_K)
 {
-    int sk = Split_K <= 0 ? SpMM_SplitK_Auto(M, N, K) : clamp_split_k(Split_K, K);
+    if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
+        return 0;
+    if (Split_K <= 0)
+        return spmm::streamk_workspace_bytes(M, N, K);
+    int sk = clamp_split_k(Split_K, K);
     if (sk <= 1)
         return 0;
     return sizeof(float) * (size_t)M * (size_t)N * (size_t)sk;
@@ -123,6 +128,22 @@ extern "C" int SpMM_SplitK_API(hipStream_t stream, const void* values, const uin
 {
     if (int e = check_shape(M, N, K))
         return e;
+    if (Split_K <= 0 && spmm::kernel_variant() == 2) {
+        // the library's own split: one persistent kernel, partial sums and arrival counters in the workspace
+        if (workspace == nullptr) {
+            std::printf("MM_Sparse_API Error: Split_K<=0 needs SpMM_WorkspaceBytes(M, N, K, 0) bytes of workspace!\n");
+            std::fflush(stdout);
+            return (int)hipErrorInvalidValue;
+        }
+        static std::atomic<unsigned> next_ticket{1};
+        (void)hipGetLastError();
+        hipEvent_t before = t_before_main, after = t_after_main;
+        t_before_main = t_after_main = nullptr;
+        spmm::launch_streamk(stream, static_cast<const __half*>(values), bitmaps, offsets,
+                             static_cast<const __half*>(X), static_cast<__half*>(C), M, N, K, workspace,
+                             next_ticket.fetch_add(1, std::memory_order_relaxed), before, after);
+        return (int)hipGetLastError();
+    }
     int sk = Split_K <= 0 ? SpMM_SplitK_Auto(M, N, K) : Split_K;
     return run(stream, values, bitmaps, offsets, X, C, M, N, K, workspace, sk, /*fp32_partials=*/true);
 }

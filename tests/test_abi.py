@@ -35,7 +35,10 @@ def test_host_only_helpers():
     assert S.SpMM_WorkspaceBytes(4096, 16, 4096, 4) == 4 * 4096 * 16 * 4
     sk = S.SpMM_SplitK_Auto(5120, 16, 5120)
     assert 1 <= sk <= 5120 // 64
-    assert S.SpMM_WorkspaceBytes(5120, 16, 5120, 0) == (0 if sk == 1 else 4 * 5120 * 16 * sk)
+    # Split_K <= 0: the persistent kernel's partial slots and arrival counters, independent of any Split_K
+    auto_bytes = S.SpMM_WorkspaceBytes(5120, 16, 5120, 0)
+    assert auto_bytes > 8 * (5120 // 64) and auto_bytes % 8 == 0
+    assert S.SpMM_WorkspaceBytes(5120, 24, 5120, 0) == 0  # unsupported N: nothing to size
 
 
 def test_shape_errors_are_reported_without_a_gpu(capfd):

@@ -190,6 +190,40 @@ def test_auto_split_k_and_invariance(torch, oracle):
         assert_spmm_close(dev.spmm(X, sk), ref, f"sk={sk}")
 
 
+@pytest.mark.parametrize("M,K,N,s", [
+    (256, 512, 16, 0.6),      # ranges of a few tiles: every row block is shared by several workgroups
+    (65536, 192, 16, 0.7),    # three tiles per row block: ranges straddle row-block boundaries
+    (8192, 128, 32, 0.5),     # two tiles per row block: whole row blocks only
+    (1024, 4096, 8, 0.7),
+    (4096, 1024, 64, 0.5),
+    (2048, 2048, 128, 0.6),   # two column blocks
+])
+def test_library_split_repeated_calls_reuse_workspace(torch, oracle, M, K, N, s):
+    """Split_K <= 0 (persistent kernel): partial slots and arrival counters live in the caller's workspace,
+    whose previous contents (garbage, or an earlier call's counters) must not matter."""
+    W = make_weight(M, K, s, seed=M + K)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    dev = Device(torch, comp)
+    nbytes = S.SpMM_WorkspaceBytes(M, N, K, 0)
+    ws = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device="cuda:0")  # garbage on purpose
+    for rep in range(3):
+        X = make_activations(K, N, seed=rep)
+        x = torch.from_numpy(X.view(np.int16).copy()).to("cuda:0")
+        out = torch.full((N, M), 0x7e00, dtype=torch.int16, device="cuda:0")
+        print(f"case M={M} K={K} N={N} rep={rep}", flush=True)
+        err = S.SpMM_SplitK_API(None, dev.values, dev.bitmaps, dev.offsets, x, out, M, N, K, ws, 0)
+        assert err == 0
+        torch.cuda.synchronize()
+        C = out.cpu().numpy().view(np.float16)
+        assert_spmm_close(C, _oracle_C(oracle, comp, X), f"rep {rep}")
+
+
+def test_library_split_needs_workspace(torch, capfd):
+    t = torch.zeros(64, dtype=torch.int16, device="cuda:0")
+    assert S.SpMM_SplitK_API(None, t, t, t, t, t, 64, 16, 64, None, 0) == S.api.HIP_ERROR_INVALID_VALUE
+    assert "workspace" in capfd.readouterr().out
+
+
 def test_linearity_at_full_size(torch):
     """OPT-13B QKV shape: C(X1 + X2) == C(X1) + C(X2) within the contract, and C(0) == 0."""
     M, K, N = 15360, 5120, 16
