@@ -53,10 +53,11 @@ typedef struct ihipEvent_t*  hipEvent_t;
  *   Split_K >= 1  use that many K batches (partition as in
  *                 csrc/SpMM_Kernel.cuh:35-43);
  *   Split_K <= 0  the library picks one for the shape (SpMM_SplitK_Auto).
- * When the effective Split_K is > 1, `workspace` must hold
- * SpMM_WorkspaceBytes(M, N, K, Split_K) bytes: partial sums are kept in fp32
- * (4*M*N*Split_K bytes) and reduced to fp16 by a second kernel.  It may be
- * NULL when the effective Split_K is 1.
+ * `workspace` must hold SpMM_WorkspaceBytes(M, N, K, Split_K) bytes (call it
+ * with the same Split_K argument, <= 0 included): partial sums are kept in
+ * fp32 (4*M*N*Split_K bytes for an explicit Split_K > 1) and reduced to fp16
+ * by a second kernel.  It may be NULL when that size is 0.  Its contents on
+ * entry do not matter.
  * Returns a hipError_t value as int: 0 on success; 999 (hipErrorUnknown) with
  * the reference's message for an unsupported N (csrc/SpMM_API.cuh:91-94);
  * 1 (hipErrorInvalidValue) for M or K not a multiple of 64 or a missing
@@ -90,8 +91,9 @@ int SpMM_SplitK_API_bitmap_v3(hipStream_t stream, const void* A, const void* Com
  */
 int SpMM_SplitK_Auto(int M, int N, int K);
 
-/* Bytes of workspace SpMM_SplitK_API needs for this call (0 when the
- * effective Split_K is 1).  Split_K <= 0 means the automatic choice. */
+/* Bytes of workspace SpMM_SplitK_API needs for this call (0 for Split_K == 1).
+ * Split_K <= 0 means the library's own choice and returns a size that covers
+ * whatever way it may split the work. */
 size_t SpMM_WorkspaceBytes(int M, int N, int K, int Split_K);
 
 /*

@@ -115,8 +115,13 @@ extern "C" size_t SpMM_WorkspaceBytes(int M, int N, int K, int Split_K)
 {
     if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
         return 0;
-    if (Split_K <= 0)
-        return spmm::streamk_workspace_bytes(M, N, K);
+    if (Split_K <= 0) {
+        // enough for either way the library may split the work itself
+        const int    sk0     = SpMM_SplitK_Auto(M, N, K);
+        const size_t classic = sk0 > 1 ? sizeof(float) * (size_t)M * (size_t)N * (size_t)sk0 : 0;
+        const size_t streamk = spmm::streamk_workspace_bytes(M, N, K);
+        return classic > streamk ? classic : streamk;
+    }
     int sk = clamp_split_k(Split_K, K);
     if (sk <= 1)
         return 0;
@@ -128,8 +133,8 @@ extern "C" int SpMM_SplitK_API(hipStream_t stream, const void* values, const uin
 {
     if (int e = check_shape(M, N, K))
         return e;
-    if (Split_K <= 0 && spmm::kernel_variant() == 2) {
-        // the library's own split: one persistent kernel, partial sums and arrival counters in the workspace
+    if (Split_K <= 0 && spmm::kernel_variant() == 3) {
+        // experimental: one persistent kernel, partial sums and arrival counters in the workspace
         if (workspace == nullptr) {
             std::printf("MM_Sparse_API Error: Split_K<=0 needs SpMM_WorkspaceBytes(M, N, K, 0) bytes of workspace!\n");
             std::fflush(stdout);

@@ -91,6 +91,19 @@ def test_matches_oracle(torch, oracle, M, K, N, s, sk):
     assert_spmm_close(Cv3, ref64, "v3 vs float64")
 
 
+@pytest.mark.parametrize("variant", ["baseline", "stream"])
+def test_other_kernel_variants_match_oracle(torch, oracle, monkeypatch, variant):
+    """The comparison kernels (simple staging kernel, lane-per-bit decode through a dense LDS tile) stay correct."""
+    monkeypatch.setenv("SPMM_KERNEL", variant)
+    for M, K, N, s, sk in [(128, 192, 16, 0.7, 1), (256, 1024, 8, 0.6, 3), (128, 512, 64, 0.5, 2), (256, 256, 32, 0.0, 1)]:
+        W = make_weight(M, K, s, seed=M + K + N)
+        X = make_activations(K, N, seed=N)
+        comp = S.InitSparseMatrixA_bitmap(W)
+        print(f"case {variant} M={M} K={K} N={N} sk={sk}", flush=True)
+        C = Device(torch, comp).spmm(X, sk, "api")
+        assert_spmm_close(C, _oracle_C(oracle, comp, X, sk, False), f"{variant} {M}x{K}x{N}")
+
+
 def test_exact_on_small_integers(torch, oracle):
     """Where fp32 accumulation is exact the result must be bit-identical to the oracle, any Split_K."""
     rng = np.random.default_rng(5)
@@ -198,9 +211,12 @@ def test_auto_split_k_and_invariance(torch, oracle):
     (4096, 1024, 64, 0.5),
     (2048, 2048, 128, 0.6),   # two column blocks
 ])
-def test_library_split_repeated_calls_reuse_workspace(torch, oracle, M, K, N, s):
-    """Split_K <= 0 (persistent kernel): partial slots and arrival counters live in the caller's workspace,
-    whose previous contents (garbage, or an earlier call's counters) must not matter."""
+@pytest.mark.parametrize("variant", ["rows", "streamk"])
+def test_library_split_repeated_calls_reuse_workspace(torch, oracle, monkeypatch, variant, M, K, N, s):
+    """Split_K <= 0: the workspace's previous contents (garbage, or an earlier call's partial sums and arrival
+    counters) must not matter, for the default kernel and for the persistent one (SPMM_KERNEL=streamk), which
+    keeps partial slots and per-row-block arrival counters there."""
+    monkeypatch.setenv("SPMM_KERNEL", variant)
     W = make_weight(M, K, s, seed=M + K)
     comp = S.InitSparseMatrixA_bitmap(W)
     dev = Device(torch, comp)
@@ -210,7 +226,7 @@ def test_library_split_repeated_calls_reuse_workspace(torch, oracle, M, K, N, s)
         X = make_activations(K, N, seed=rep)
         x = torch.from_numpy(X.view(np.int16).copy()).to("cuda:0")
         out = torch.full((N, M), 0x7e00, dtype=torch.int16, device="cuda:0")
-        print(f"case M={M} K={K} N={N} rep={rep}", flush=True)
+        print(f"case {variant} M={M} K={K} N={N} rep={rep}", flush=True)
         err = S.SpMM_SplitK_API(None, dev.values, dev.bitmaps, dev.offsets, x, out, M, N, K, ws, 0)
         assert err == 0
         torch.cuda.synchronize()
@@ -218,9 +234,15 @@ def test_library_split_repeated_calls_reuse_workspace(torch, oracle, M, K, N, s)
         assert_spmm_close(C, _oracle_C(oracle, comp, X), f"rep {rep}")
 
 
-def test_library_split_needs_workspace(torch, capfd):
+def test_library_split_needs_workspace(torch, capfd, monkeypatch):
+    """A missing workspace is reported before anything is launched."""
     t = torch.zeros(64, dtype=torch.int16, device="cuda:0")
+    monkeypatch.setenv("SPMM_KERNEL", "streamk")
     assert S.SpMM_SplitK_API(None, t, t, t, t, t, 64, 16, 64, None, 0) == S.api.HIP_ERROR_INVALID_VALUE
+    assert "workspace" in capfd.readouterr().out
+    monkeypatch.delenv("SPMM_KERNEL")
+    assert S.SpMM_WorkspaceBytes(512, 16, 4096, 0) > 0
+    assert S.SpMM_SplitK_API(None, t, t, t, t, t, 512, 16, 4096, None, 0) == S.api.HIP_ERROR_INVALID_VALUE
     assert "workspace" in capfd.readouterr().out
 
 
