@@ -40,6 +40,8 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-dense", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    p.add_argument("--copy-probe", action="store_true",
+                   help="also run three 256 MiB device-to-device copies (a known-size reference for HBM byte counters)")
     return p.parse_args()
 
 
@@ -177,6 +179,14 @@ def main():
     for e0, e1 in events:
         hip.rt.hipEventDestroy(e0), hip.rt.hipEventDestroy(e1)
 
+    if a.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     ms_per_step = wall / a.steps * 1e3
     flops = 2.0 * M * N * K
     value = flops / (wall / a.steps) / 1e12
@@ -206,6 +216,13 @@ def main():
                  "what": "torch.matmul fp16 (hipBLASLt), same run, rotating weight copies"}
         del Wd
 
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):  # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+        rec = json.load(open(tpath)).get(f"{a.workload}_n{N}_s{int(round(w['sparsity'] * 100))}")
+        if rec:
+            traffic = rec["bytes_per_launch"]
+
     out = {
         "metric": "SpMM dense-equiv TFLOP/s", "value": value, "unit": "TFLOP/s", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
@@ -217,7 +234,7 @@ def main():
                    "workspace_bytes": ws_bytes},
         "gbs_whole_call": algo_bytes / (wall / a.steps) / 1e9,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes_per_launch": algo_bytes, "kernel": "spmm main kernel",
                      "kernel_avg_us": kern_avg_s * 1e6, "kernel_min_us": float(kern_ms.min()) * 1e3,
                      "timing": "HIP events attached to each main-kernel dispatch (kernel begin/end timestamps), "
