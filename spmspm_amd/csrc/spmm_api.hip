@@ -3,7 +3,6 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
-#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 
@@ -134,19 +133,18 @@ extern "C" int SpMM_SplitK_API(hipStream_t stream, const void* values, const uin
     if (int e = check_shape(M, N, K))
         return e;
     if (Split_K <= 0 && spmm::kernel_variant() == 3) {
-        // experimental: one persistent kernel, partial sums and arrival counters in the workspace
+        // one persistent kernel plus a fix-up kernel, partial sums in the workspace
         if (workspace == nullptr) {
             std::printf("MM_Sparse_API Error: Split_K<=0 needs SpMM_WorkspaceBytes(M, N, K, 0) bytes of workspace!\n");
             std::fflush(stdout);
             return (int)hipErrorInvalidValue;
         }
-        static std::atomic<unsigned> next_ticket{1};
         (void)hipGetLastError();
         hipEvent_t before = t_before_main, after = t_after_main;
         t_before_main = t_after_main = nullptr;
         spmm::launch_streamk(stream, static_cast<const __half*>(values), bitmaps, offsets,
-                             static_cast<const __half*>(X), static_cast<__half*>(C), M, N, K, workspace,
-                             next_ticket.fetch_add(1, std::memory_order_relaxed), before, after);
+                             static_cast<const __half*>(X), static_cast<__half*>(C), M, N, K, workspace, before,
+                             after);
         return (int)hipGetLastError();
     }
     int sk = Split_K <= 0 ? SpMM_SplitK_Auto(M, N, K) : Split_K;
