@@ -114,14 +114,7 @@ extern "C" size_t SpMM_WorkspaceBytes(int M, int N, int K, int Split_K)
 {
     if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
         return 0;
-    if (Split_K <= 0) {
-        // enough for either way the library may split the work itself
-        const int    sk0     = SpMM_SplitK_Auto(M, N, K);
-        const size_t classic = sk0 > 1 ? sizeof(float) * (size_t)M * (size_t)N * (size_t)sk0 : 0;
-        const size_t streamk = spmm::streamk_workspace_bytes(M, N, K);
-        return classic > streamk ? classic : streamk;
-    }
-    int sk = clamp_split_k(Split_K, K);
+    int sk = clamp_split_k(Split_K <= 0 ? auto_split_k(M, N, K) : Split_K, K);
     if (sk <= 1)
         return 0;
     return sizeof(float) * (size_t)M * (size_t)N * (size_t)sk;
@@ -132,21 +125,6 @@ extern "C" int SpMM_SplitK_API(hipStream_t stream, const void* values, const uin
 {
     if (int e = check_shape(M, N, K))
         return e;
-    if (Split_K <= 0 && spmm::kernel_variant() == 3) {
-        // one persistent kernel plus a fix-up kernel, partial sums in the workspace
-        if (workspace == nullptr) {
-            std::printf("MM_Sparse_API Error: Split_K<=0 needs SpMM_WorkspaceBytes(M, N, K, 0) bytes of workspace!\n");
-            std::fflush(stdout);
-            return (int)hipErrorInvalidValue;
-        }
-        (void)hipGetLastError();
-        hipEvent_t before = t_before_main, after = t_after_main;
-        t_before_main = t_after_main = nullptr;
-        spmm::launch_streamk(stream, static_cast<const __half*>(values), bitmaps, offsets,
-                             static_cast<const __half*>(X), static_cast<__half*>(C), M, N, K, workspace, before,
-                             after);
-        return (int)hipGetLastError();
-    }
     int sk = Split_K <= 0 ? SpMM_SplitK_Auto(M, N, K) : Split_K;
     return run(stream, values, bitmaps, offsets, X, C, M, N, K, workspace, sk, /*fp32_partials=*/true);
 }

@@ -204,19 +204,16 @@ def test_auto_split_k_and_invariance(torch, oracle):
 
 
 @pytest.mark.parametrize("M,K,N,s", [
-    (256, 512, 16, 0.6),      # ranges of a few tiles: every row block is shared by several workgroups
-    (65536, 192, 16, 0.7),    # three tiles per row block: ranges straddle row-block boundaries
-    (8192, 128, 32, 0.5),     # two tiles per row block: whole row blocks only
+    (256, 512, 16, 0.6),
+    (65536, 192, 16, 0.7),    # three group tiles per row block
+    (8192, 128, 32, 0.5),     # two group tiles per row block
     (1024, 4096, 8, 0.7),
     (4096, 1024, 64, 0.5),
     (2048, 2048, 128, 0.6),   # two column blocks
 ])
-@pytest.mark.parametrize("variant", ["rows", "streamk"])
-def test_library_split_repeated_calls_reuse_workspace(torch, oracle, monkeypatch, variant, M, K, N, s):
-    """Split_K <= 0: the workspace's previous contents (garbage, or an earlier call's partial sums and arrival
-    counters) must not matter, for the default kernel and for the persistent one (SPMM_KERNEL=streamk), which
-    keeps partial slots and per-row-block arrival counters there."""
-    monkeypatch.setenv("SPMM_KERNEL", variant)
+def test_library_split_repeated_calls_reuse_workspace(torch, oracle, M, K, N, s):
+    """Split_K <= 0: the workspace's previous contents (garbage, or an earlier call's partial sums) must not
+    matter."""
     W = make_weight(M, K, s, seed=M + K)
     comp = S.InitSparseMatrixA_bitmap(W)
     dev = Device(torch, comp)
@@ -226,7 +223,7 @@ def test_library_split_repeated_calls_reuse_workspace(torch, oracle, monkeypatch
         X = make_activations(K, N, seed=rep)
         x = torch.from_numpy(X.view(np.int16).copy()).to("cuda:0")
         out = torch.full((N, M), 0x7e00, dtype=torch.int16, device="cuda:0")
-        print(f"case {variant} M={M} K={K} N={N} rep={rep}", flush=True)
+        print(f"case M={M} K={K} N={N} rep={rep}", flush=True)
         err = S.SpMM_SplitK_API(None, dev.values, dev.bitmaps, dev.offsets, x, out, M, N, K, ws, 0)
         assert err == 0
         torch.cuda.synchronize()
@@ -234,13 +231,9 @@ def test_library_split_repeated_calls_reuse_workspace(torch, oracle, monkeypatch
         assert_spmm_close(C, _oracle_C(oracle, comp, X), f"rep {rep}")
 
 
-def test_library_split_needs_workspace(torch, capfd, monkeypatch):
+def test_library_split_needs_workspace(torch, capfd):
     """A missing workspace is reported before anything is launched."""
     t = torch.zeros(64, dtype=torch.int16, device="cuda:0")
-    monkeypatch.setenv("SPMM_KERNEL", "streamk")
-    assert S.SpMM_SplitK_API(None, t, t, t, t, t, 64, 16, 64, None, 0) == S.api.HIP_ERROR_INVALID_VALUE
-    assert "workspace" in capfd.readouterr().out
-    monkeypatch.delenv("SPMM_KERNEL")
     assert S.SpMM_WorkspaceBytes(512, 16, 4096, 0) > 0
     assert S.SpMM_SplitK_API(None, t, t, t, t, t, 512, 16, 4096, None, 0) == S.api.HIP_ERROR_INVALID_VALUE
     assert "workspace" in capfd.readouterr().out
