@@ -40,6 +40,9 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-dense", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    p.add_argument("--no-chain", action="store_true",
+                   help="skip the OPT-13B decode-step chain (40 layers x 4 linears, sparse vs dense, same run)")
+    p.add_argument("--chain-layers", type=int, default=40)
     p.add_argument("--copy-probe", action="store_true",
                    help="also run three 256 MiB device-to-device copies (a known-size reference for HBM byte counters)")
     return p.parse_args()
@@ -106,6 +109,85 @@ def cpu_baseline(comp, X, seconds):
         "seconds_per_pass": t, "passes": reps,
         "encoder_melems_per_s_1thread": enc_rows * K / t_enc / 1e6,
     }
+
+
+def decode_chain(torch, S, dev, layers, seed):
+    """OPT-13B decode step, linears only: `layers` x {QKV, out, FFN1, FFN2} at N=16, every layer with weight
+    copies of its own, chained on one stream (FFN2's output feeds the next layer's QKV; the attention between QKV
+    and the output projection is not run, its result is a fixed buffer).  Timed eagerly and as a replayed HIP
+    graph, for the compressed weights and for dense fp16 weights (torch.matmul) in the same run."""
+    from spmspm_amd.synthetic import WORKLOADS, make_weight
+    N = 16
+    names = ["opt13b_qkv", "opt13b_out", "opt13b_ffn1", "opt13b_ffn2"]
+    first, dense0, info = [], [], []
+    for i, nm in enumerate(names):
+        w = WORKLOADS[nm]
+        W = make_weight(w["M"], w["K"], w["sparsity"], seed=seed + 11 * i, pruning=w["pruning"])
+        comp = S.InitSparseMatrixA_bitmap(W)
+        first.append(S.SparseLinear(comp, device=dev, split_k=0))
+        dense0.append(torch.from_numpy(W.view(np.int16)).to(dev).view(torch.float16))
+        info.append({"name": nm, "M": w["M"], "K": w["K"], "sparsity": w["sparsity"],
+                     "split_k": S.SpMM_SplitK_Auto(w["M"], N, w["K"]), "bytes": comp.algorithmic_bytes(N)})
+        del W, comp
+    sparse = [[l if j == 0 else l.clone() for l in first] for j in range(layers)]
+    dense = [[d if j == 0 else d.clone() for d in dense0] for j in range(layers)]
+    for row in sparse:
+        for l in row:
+            l.workspace(N)
+    h = (torch.rand((N, 5120), device=dev) * 2 - 1).to(torch.float16)
+    attn = (torch.rand((N, 5120), device=dev) * 2 - 1).to(torch.float16)
+    qkv = torch.empty((N, 15360), dtype=torch.float16, device=dev)
+    o = torch.empty((N, 5120), dtype=torch.float16, device=dev)
+    f = torch.empty((N, 20480), dtype=torch.float16, device=dev)
+    hs = [torch.empty((N, 5120), dtype=torch.float16, device=dev) for _ in range(2)]
+
+    def run_sparse(stream):
+        x = h
+        for j, (lq, lo, l1, l2) in enumerate(sparse):
+            lq(x, out=qkv, stream=stream)
+            lo(attn, out=o, stream=stream)
+            l1(o, out=f, stream=stream)
+            x = l2(f, out=hs[j & 1], stream=stream)
+
+    def run_dense(stream):
+        x = h
+        for j, (wq, wo, w1, w2) in enumerate(dense):
+            torch.matmul(x, wq.t(), out=qkv)
+            torch.matmul(attn, wo.t(), out=o)
+            torch.matmul(o, w1.t(), out=f)
+            x = torch.matmul(f, w2.t(), out=hs[j & 1])
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps * 1e3
+
+    out = {"layers": layers, "N": N, "linears": info, "calls_per_step": 4 * layers,
+           "what": "ms per decode step over the linears of all layers; weights of every layer resident separately"}
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        out["sparse_eager_ms"] = timed(lambda: run_sparse(side), 5)
+        out["dense_eager_ms"] = timed(lambda: run_dense(side), 5)
+        for name, fn in (("sparse", run_sparse), ("dense", run_dense)):
+            try:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=side):
+                    fn(side)
+                out[name + "_graph_ms"] = timed(g.replay, 10)
+            except Exception as e:  # capture is an extra; the eager figures stand on their own
+                out[name + "_graph_ms"] = None
+                out[name + "_graph_error"] = str(e)[:200]
+    torch.cuda.synchronize()
+    sp = out.get("sparse_graph_ms") or out["sparse_eager_ms"]
+    de = out.get("dense_graph_ms") or out["dense_eager_ms"]
+    out["speedup_vs_dense"] = de / sp
+    out["weight_bytes_sparse"] = int(sum(i["bytes"] for i in info)) * layers
+    out["weight_bytes_dense"] = int(sum(2 * i["M"] * i["K"] for i in info)) * layers
+    return out
 
 
 def main():
@@ -243,6 +325,10 @@ def main():
         "dense_fp16": dense,
         "host": {"generate_s": t_gen, "encode_s": t_enc, "encode_threads": os.cpu_count()},
     }
+    if not a.no_chain:
+        del layers, xs, outs
+        torch.cuda.empty_cache()
+        out["decode_chain_opt13b"] = decode_chain(torch, S, dev, a.chain_layers, a.seed)
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(comp, X, a.cpu_seconds)
     print(json.dumps(out))

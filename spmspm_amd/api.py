@@ -231,6 +231,13 @@ class SparseLinear:
         self.split_k = split_k
         self._ws = None
 
+    def clone(self):
+        """A second resident copy of the same weights (device-to-device), e.g. one per decoder layer."""
+        c = object.__new__(SparseLinear)
+        c.M, c.K, c.device, c.nnz_padded, c.split_k, c._ws = self.M, self.K, self.device, self.nnz_padded, self.split_k, None
+        c.values, c.bitmaps, c.offsets = self.values.clone(), self.bitmaps.clone(), self.offsets.clone()
+        return c
+
     def bytes_per_call(self, N):
         return (2 * self.nnz_padded + 8 * self.bitmaps.numel() + 4 * self.offsets.numel()
                 + 2 * self.K * N + 2 * self.M * N)

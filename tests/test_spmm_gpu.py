@@ -291,3 +291,48 @@ def test_stream_argument_is_honoured(torch, oracle):
         y = lin(x, stream=side)
     side.synchronize()
     assert_spmm_close(y.cpu().numpy(), _oracle_C(oracle, comp, X, 2), "side stream")
+
+
+def test_calls_recorded_in_a_hip_graph_replay_correctly(torch, oracle):
+    """Three chained SpMM calls (split and unsplit) captured from a stream and replayed: every replay, with eager
+    work and synchronisations of the program's own in between, must give what the eager chain gives."""
+    M, K, N = 512, 512, 16
+    comps = [S.InitSparseMatrixA_bitmap(make_weight(M, K, 0.6, seed=40 + i)) for i in range(3)]
+    lins = [S.SparseLinear(c, split_k=sk) for c, sk in zip(comps, (1, 4, 0))]
+    for l in lins:
+        l.workspace(N)
+    x0 = torch.zeros((N, K), dtype=torch.float16, device="cuda:0")
+    bufs = [torch.empty((N, M), dtype=torch.float16, device="cuda:0") for _ in range(3)]
+
+    def chain(stream):
+        x = x0
+        for l, b in zip(lins, bufs):
+            x = l(x, out=b, stream=stream)
+
+    def expected(X):
+        x = X
+        for c, sk in zip(comps, (1, 4, S.SpMM_SplitK_Auto(M, N, K))):
+            x = oracle.spmm(c.values, c.bitmaps, c.offsets, x, M, N, K, sk, False)
+        return x
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        chain(side)  # warm-up outside the capture
+        side.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            chain(side)
+        for rep in range(4):
+            X = (make_activations(K, N, seed=100 + rep).astype(np.float32) * 8).astype(np.float16)
+            x0.copy_(torch.from_numpy(X.view(np.int16).copy()).to("cuda:0").view(torch.float16))
+            for b in bufs:
+                b.fill_(float("nan"))
+            print(f"graph replay {rep}", flush=True)
+            g.replay()
+            side.synchronize()
+            got = bufs[2].cpu().numpy()
+            assert_spmm_close(got, expected(X), f"replay {rep}")
+            chain(side)  # eager work between replays
+            side.synchronize()
+            assert np.array_equal(got.view(np.uint16), bufs[2].cpu().numpy().view(np.uint16)), "eager != replay"
