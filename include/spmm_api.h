@@ -97,6 +97,22 @@ int SpMM_SplitK_Auto(int M, int N, int K);
 size_t SpMM_WorkspaceBytes(int M, int N, int K, int Split_K);
 
 /*
+ * SpMM with bias and activation folded into the output pass:
+ *   C[m + n*M] = fp16( act( sum_k W[m][k] * X[k][n]  +  bias[m] ) ),   everything before the cast in fp32.
+ * Takes the place of the SpMM call followed by the element-wise add-bias / activation kernels of the reference's
+ * FasterTransformer layer (third_party/ft_spinfer.patch:766-768 and the unpatched FfnLayer code around it); no
+ * such entry point exists in the reference's library.  `bias` is M fp16 values on the device, or NULL.
+ * `activation`: 0 none, 1 ReLU, 2 GELU in its tanh form 0.5*x*(1 + tanh(0.79788456*(x + 0.044715*x^3))).
+ * The partial sums always pass through `workspace` (fp32), which must hold
+ * SpMM_WorkspaceBytesBiasAct(M, N, K, Split_K) bytes = 4*M*N*max(Split_K, 1), also for an unsplit K.
+ * Other arguments, Split_K <= 0 and return values as for SpMM_SplitK_API; an unknown activation returns 1.
+ */
+int SpMM_SplitK_API_BiasAct(hipStream_t stream, const void* values, const uint64_t* bitmaps, const int* offsets,
+                            const void* X, void* C, int M, int N, int K, void* workspace, int Split_K,
+                            const void* bias, int activation);
+size_t SpMM_WorkspaceBytesBiasAct(int M, int N, int K, int Split_K);
+
+/*
  * Host encoder, C twin of InitSparseMatrixA_bitmap
  * (csrc/SpMM_API.cuh:112-241): dense row-major fp16 W -> TCA-BME arrays.
  * Output is bit-identical to the reference's.  The tile-size arguments are

@@ -51,6 +51,7 @@ def lib():
         L.oracle_splitk_range.restype = C.c_int
         L.oracle_splitk_range.argtypes = [C.c_int, C.c_int, C.c_int, _i32p]
         L.oracle_spmm.argtypes = [C.c_void_p] * 5 + [C.c_int] * 5
+        L.oracle_spmm_bias_act.argtypes = [C.c_void_p] * 5 + [C.c_int] * 5 + [C.c_void_p, C.c_int]
         L.oracle_num_threads.restype = C.c_int
         L.oracle_gemm_f64.argtypes = [C.c_void_p] * 3 + [C.c_int] * 3
         L.oracle_init_host_matrices.argtypes = [C.c_void_p, C.c_void_p] + [C.c_int] * 5
@@ -155,6 +156,24 @@ def spmm(values, bitmap, global_off, X, M, N, K, split_k=1, partial_fp16=False):
     Cout = np.empty((N, M), np.uint16)
     lib().oracle_spmm(values.ctypes.data, bitmap.ctypes.data, global_off.ctypes.data, X.ctypes.data,
                       Cout.ctypes.data, M, N, K, int(split_k), int(bool(partial_fp16)))
+    return Cout.view(np.float16)
+
+
+def spmm_bias_act(values, bitmap, global_off, X, M, N, K, split_k=1, bias=None, act=0):
+    """Host SpMM with C = fp16(act(sum + bias[m])); bias: M fp16 values or None; act 0 none, 1 ReLU, 2 GELU."""
+    values = _as_u16(values)
+    if values.size == 0:
+        values = np.zeros(1, np.uint16)
+    bitmap = np.ascontiguousarray(bitmap, dtype=np.uint64)
+    global_off = np.ascontiguousarray(global_off, dtype=np.int32)
+    X = _as_u16(X)
+    assert X.size == N * K
+    b = None if bias is None else _as_u16(bias)
+    assert b is None or b.size == M
+    Cout = np.empty((N, M), np.uint16)
+    lib().oracle_spmm_bias_act(values.ctypes.data, bitmap.ctypes.data, global_off.ctypes.data, X.ctypes.data,
+                               Cout.ctypes.data, M, N, K, int(split_k), 0,
+                               None if b is None else b.ctypes.data, int(act))
     return Cout.view(np.float16)
 
 

@@ -23,6 +23,10 @@
  *                          with the reference kernel's own output bits is
  *                          unpinned; the contract is the tolerance
  *                          max|d| <= 1e-2*max|C|, rel-L2 <= 1e-3.
+ *   oracle_spmm_bias_act   the same product with bias and activation applied in
+ *                          fp32 before the rounding; pinned against float64
+ *                          numpy (relu / tanh-form gelu of GEMM + bias) and the
+ *                          functions' closed-form properties.
  *   oracle_splitk_*        pinned: partition closed form + sum over batches
  *                          equals the unsplit product.
  *   oracle_init_host_matrices  pinned: reproduces the seven recorded
@@ -284,8 +288,21 @@ int oracle_splitk_range(int K, int split_k, int batch, int* count)
  * The accumulation order inside a batch is ascending k (the kernel's order is
  * an implementation detail; the tolerance in the tests absorbs it).
  */
-void oracle_spmm(const uint16_t* vals, const uint64_t* bitmap, const int* global, const uint16_t* X,
-                 uint16_t* C, int M, int N, int K, int split_k, int partial_fp16)
+/* act: 0 none, 1 ReLU, 2 GELU (tanh form, as FasterTransformer's gelu) */
+static float oracle_activation(float x, int act)
+{
+    if (act == 1)
+        return x > 0.f ? x : (x == x ? 0.f : x);
+    if (act == 2)
+        return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+    return x;
+}
+
+/* SpMM with the element-wise tail of the reference's FfnLayer folded in before the fp16 rounding
+ * (third_party/ft_spinfer.patch:766-768): C = fp16(act(sum + bias[m])).  bias may be NULL. */
+void oracle_spmm_bias_act(const uint16_t* vals, const uint64_t* bitmap, const int* global, const uint16_t* X,
+                          uint16_t* C, int M, int N, int K, int split_k, int partial_fp16, const uint16_t* bias,
+                          int act)
 {
     if (split_k < 1)
         split_k = 1;
@@ -336,10 +353,21 @@ void oracle_spmm(const uint16_t* vals, const uint64_t* bitmap, const int* global
             }
             for (int n = 0; n < N; ++n)
                 for (int r = 0; r < 64; ++r)
-                    C[(size_t)n * M + gm * 64 + r] = oracle_float_to_half(tot[n * 64 + r]);
+                {
+                    float v = tot[n * 64 + r];
+                    if (bias)
+                        v += oracle_half_to_float(bias[gm * 64 + r]);
+                    C[(size_t)n * M + gm * 64 + r] = oracle_float_to_half(oracle_activation(v, act));
+                }
         }
         free(wrow), free(xt), free(acc), free(tot);
     }
+}
+
+void oracle_spmm(const uint16_t* vals, const uint64_t* bitmap, const int* global, const uint16_t* X,
+                 uint16_t* C, int M, int N, int K, int split_k, int partial_fp16)
+{
+    oracle_spmm_bias_act(vals, bitmap, global, X, C, M, N, K, split_k, partial_fp16, NULL, 0);
 }
 
 int oracle_num_threads(void)

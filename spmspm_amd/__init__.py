@@ -9,7 +9,12 @@ from .api import (  # noqa: F401
     InitSparseMatrixA_bitmap,
     Our_GenSparseMatrixBinFile,
     SparseLinear,
+    ACT_GELU,
+    ACT_NONE,
+    ACT_RELU,
     SpMM_SplitK_API,
+    SpMM_SplitK_API_BiasAct,
+    SpMM_WorkspaceBytesBiasAct,
     SpMM_SplitK_API_bitmap_v3,
     SpMM_SplitK_Auto,
     SpMM_WorkspaceBytes,

@@ -46,6 +46,10 @@ def library():
     L.SpMM_SplitK_Auto.argtypes = [C.c_int] * 3
     L.SpMM_WorkspaceBytes.restype = C.c_size_t
     L.SpMM_WorkspaceBytes.argtypes = [C.c_int] * 4
+    L.SpMM_SplitK_API_BiasAct.restype = C.c_int
+    L.SpMM_SplitK_API_BiasAct.argtypes = [C.c_void_p] * 6 + [C.c_int] * 3 + [C.c_void_p, C.c_int, C.c_void_p, C.c_int]
+    L.SpMM_WorkspaceBytesBiasAct.restype = C.c_size_t
+    L.SpMM_WorkspaceBytesBiasAct.argtypes = [C.c_int] * 4
     L.InitSparseMatrixA_bitmap.restype = C.c_int
     L.InitSparseMatrixA_bitmap.argtypes = [C.c_void_p] + [C.c_int] * 8 + [
         C.POINTER(_u16p), C.POINTER(_i32p), C.POINTER(_i32p), C.POINTER(_i32p), C.POINTER(_u64p), _i32p]
@@ -201,6 +205,20 @@ def SpMM_SplitK_API(stream, values, bitmaps, offsets, X, C_out, M, N, K, workspa
                                      _ptr(C_out), M, N, K, _ptr(workspace), Split_K)
 
 
+ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
+
+
+def SpMM_WorkspaceBytesBiasAct(M, N, K, Split_K):
+    return int(library().SpMM_WorkspaceBytesBiasAct(M, N, K, Split_K))
+
+
+def SpMM_SplitK_API_BiasAct(stream, values, bitmaps, offsets, X, C_out, M, N, K, workspace, Split_K, bias, activation):
+    """C = act(W*X + bias) with the tail applied in fp32 before the fp16 rounding (include/spmm_api.h)."""
+    return library().SpMM_SplitK_API_BiasAct(_stream_handle(stream), _ptr(values), _ptr(bitmaps), _ptr(offsets),
+                                             _ptr(X), _ptr(C_out), M, N, K, _ptr(workspace), Split_K, _ptr(bias),
+                                             int(activation))
+
+
 def SpMM_SplitK_API_bitmap_v3(stream, A, Compressed_A, TileOffsets, TileOffsets_Median, bitmap, max_nnz_intile, B,
                               C_out, M_Global, N_Global, K_Global, Reduction_Workspace, Split_K):
     """The reference's 14-argument call (kernel_benchmark/spmm_test.cu:375-388).  Returns the hipError_t."""
@@ -218,10 +236,21 @@ class SparseLinear:
     x: [N][K] fp16 on the device; returns [N][M] fp16.
     """
 
-    def __init__(self, compressed, device="cuda:0", split_k=0):
+    def __init__(self, compressed, device="cuda:0", split_k=0, bias=None, activation=ACT_NONE):
+        """bias: M fp16 values (numpy or tensor) added to every output column; activation: ACT_NONE/RELU/GELU.
+        With either, calls go through SpMM_SplitK_API_BiasAct."""
         import torch
         self.M, self.K = compressed.M, compressed.K
         self.device = torch.device(device)
+        self.activation = int(activation)
+        if bias is None:
+            self.bias = None
+        elif isinstance(bias, np.ndarray):
+            self.bias = torch.from_numpy(np.ascontiguousarray(bias, np.float16).view(np.int16)).to(self.device)
+        else:
+            self.bias = bias.to(self.device).contiguous()
+        if self.bias is not None and self.bias.numel() != self.M:
+            raise ValueError("bias must have M elements")
         nnz = compressed.values.size
         vals = compressed.values if nnz else np.zeros(8, np.uint16)
         self.values = torch.from_numpy(vals.view(np.int16)).to(self.device)
@@ -235,6 +264,7 @@ class SparseLinear:
         """A second resident copy of the same weights (device-to-device), e.g. one per decoder layer."""
         c = object.__new__(SparseLinear)
         c.M, c.K, c.device, c.nnz_padded, c.split_k, c._ws = self.M, self.K, self.device, self.nnz_padded, self.split_k, None
+        c.activation, c.bias = self.activation, (None if self.bias is None else self.bias.clone())
         c.values, c.bitmaps, c.offsets = self.values.clone(), self.bitmaps.clone(), self.offsets.clone()
         return c
 
@@ -244,7 +274,8 @@ class SparseLinear:
 
     def workspace(self, N):
         import torch
-        need = SpMM_WorkspaceBytes(self.M, N, self.K, self.split_k)
+        fused = self.bias is not None or self.activation != ACT_NONE
+        need = (SpMM_WorkspaceBytesBiasAct if fused else SpMM_WorkspaceBytes)(self.M, N, self.K, self.split_k)
         if need == 0:
             return None
         if self._ws is None or self._ws.numel() < need:
@@ -258,8 +289,12 @@ class SparseLinear:
             raise ValueError("x must be a contiguous [N][K] fp16 tensor")
         if out is None:
             out = torch.empty((N, self.M), dtype=torch.float16, device=self.device)
-        err = SpMM_SplitK_API(stream, self.values, self.bitmaps, self.offsets, x, out, self.M, N, self.K,
-                              self.workspace(N), self.split_k)
+        if self.bias is not None or self.activation != ACT_NONE:
+            err = SpMM_SplitK_API_BiasAct(stream, self.values, self.bitmaps, self.offsets, x, out, self.M, N, self.K,
+                                          self.workspace(N), self.split_k, self.bias, self.activation)
+        else:
+            err = SpMM_SplitK_API(stream, self.values, self.bitmaps, self.offsets, x, out, self.M, N, self.K,
+                                  self.workspace(N), self.split_k)
         if err != HIP_SUCCESS:
-            raise RuntimeError(f"SpMM_SplitK_API failed with hipError_t {err}")
+            raise RuntimeError(f"SpMM call failed with hipError_t {err}")
         return out

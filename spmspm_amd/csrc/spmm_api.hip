@@ -79,12 +79,13 @@ thread_local hipEvent_t t_before_main = nullptr;
 thread_local hipEvent_t t_after_main  = nullptr;
 
 int run(hipStream_t stream, const void* values, const uint64_t* bitmaps, const int* offsets, const void* X, void* C,
-        int M, int N, int K, void* workspace, int split_k, bool fp32_partials)
+        int M, int N, int K, void* workspace, int split_k, bool fp32_partials, bool epilogue = false,
+        const void* bias = nullptr, int act = 0)
 {
     if (int e = check_shape(M, N, K))
         return e;
     split_k = clamp_split_k(split_k, K);
-    if (split_k > 1 && workspace == nullptr) {
+    if ((split_k > 1 || epilogue) && workspace == nullptr) {
         std::printf("MM_Sparse_API Error: Split_K=%d needs a reduction workspace!\n", split_k);
         std::fflush(stdout);
         return (int)hipErrorInvalidValue;
@@ -93,11 +94,11 @@ int run(hipStream_t stream, const void* values, const uint64_t* bitmaps, const i
     hipEvent_t before = t_before_main, after = t_after_main;
     t_before_main = t_after_main = nullptr;
     spmm::launch_spmm(stream, static_cast<const __half*>(values), bitmaps, offsets, static_cast<const __half*>(X),
-                      static_cast<__half*>(C), M, N, K, workspace, split_k, fp32_partials, before, after);
+                      static_cast<__half*>(C), M, N, K, workspace, split_k, fp32_partials, before, after, epilogue);
     hipError_t err = hipGetLastError();
-    if (err != hipSuccess || split_k == 1)
+    if (err != hipSuccess || (split_k == 1 && !epilogue))
         return (int)err;
-    spmm::launch_reduction(stream, static_cast<__half*>(C), workspace, M, N, split_k, fp32_partials);
+    spmm::launch_reduction(stream, static_cast<__half*>(C), workspace, M, N, split_k, fp32_partials, bias, act);
     return (int)hipGetLastError();
 }
 
@@ -127,6 +128,30 @@ extern "C" int SpMM_SplitK_API(hipStream_t stream, const void* values, const uin
         return e;
     int sk = Split_K <= 0 ? SpMM_SplitK_Auto(M, N, K) : Split_K;
     return run(stream, values, bitmaps, offsets, X, C, M, N, K, workspace, sk, /*fp32_partials=*/true);
+}
+
+extern "C" size_t SpMM_WorkspaceBytesBiasAct(int M, int N, int K, int Split_K)
+{
+    if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
+        return 0;
+    int sk = clamp_split_k(Split_K <= 0 ? auto_split_k(M, N, K) : Split_K, K);
+    return sizeof(float) * (size_t)M * (size_t)N * (size_t)sk; // one fp32 slab even for an unsplit K
+}
+
+extern "C" int SpMM_SplitK_API_BiasAct(hipStream_t stream, const void* values, const uint64_t* bitmaps,
+                                       const int* offsets, const void* X, void* C, int M, int N, int K,
+                                       void* workspace, int Split_K, const void* bias, int activation)
+{
+    if (int e = check_shape(M, N, K))
+        return e;
+    if (activation < 0 || activation > 2) {
+        std::printf("MM_Sparse_API Error: unknown activation %d (0 none, 1 ReLU, 2 GELU)!\n", activation);
+        std::fflush(stdout);
+        return (int)hipErrorInvalidValue;
+    }
+    int sk = Split_K <= 0 ? SpMM_SplitK_Auto(M, N, K) : Split_K;
+    return run(stream, values, bitmaps, offsets, X, C, M, N, K, workspace, sk, /*fp32_partials=*/true,
+               /*epilogue=*/true, bias, activation);
 }
 
 extern "C" int SpMM_SplitK_API_bitmap_v3(hipStream_t stream, const void* /*A*/, const void* Compressed_A,

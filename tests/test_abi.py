@@ -18,7 +18,8 @@ def _declared_functions():
 def test_header_declares_the_expected_entry_points():
     names = _declared_functions()
     for n in ("SpMM_SplitK_API", "SpMM_SplitK_API_bitmap_v3", "InitSparseMatrixA_bitmap",
-              "Our_GenSparseMatrixBinFile", "SpMM_SplitK_Auto", "SpMM_WorkspaceBytes", "SpMM_Version", "SpMM_TimeNextCall"):
+              "Our_GenSparseMatrixBinFile", "SpMM_SplitK_Auto", "SpMM_WorkspaceBytes", "SpMM_Version", "SpMM_TimeNextCall",
+              "SpMM_SplitK_API_BiasAct", "SpMM_WorkspaceBytesBiasAct"):
         assert n in names
 
 
@@ -35,9 +36,11 @@ def test_host_only_helpers():
     assert S.SpMM_WorkspaceBytes(4096, 16, 4096, 4) == 4 * 4096 * 16 * 4
     sk = S.SpMM_SplitK_Auto(5120, 16, 5120)
     assert 1 <= sk <= 5120 // 64
-    # Split_K <= 0: the persistent kernel's partial slots and arrival counters, independent of any Split_K
-    auto_bytes = S.SpMM_WorkspaceBytes(5120, 16, 5120, 0)
-    assert auto_bytes > 8 * (5120 // 64) and auto_bytes % 8 == 0
+    # Split_K <= 0: sized for the library's own choice
+    assert S.SpMM_WorkspaceBytes(5120, 16, 5120, 0) == 4 * 5120 * 16 * sk
+    # with bias/activation the partial sums always pass through the workspace
+    assert S.SpMM_WorkspaceBytesBiasAct(4096, 16, 4096, 1) == 4 * 4096 * 16
+    assert S.SpMM_WorkspaceBytesBiasAct(5120, 16, 5120, 0) == 4 * 5120 * 16 * sk
     assert S.SpMM_WorkspaceBytes(5120, 24, 5120, 0) == 0  # unsupported N: nothing to size
 
 
@@ -48,3 +51,5 @@ def test_shape_errors_are_reported_without_a_gpu(capfd):
     assert S.SpMM_SplitK_API(0, 0, 0, 0, 0, 0, 100, 16, 64, 0, 1) == 1
     assert S.SpMM_SplitK_API_bitmap_v3(0, 0, 0, 0, 0, 0, 0, 0, 0, 64, 16, 64, 0, 0) == 1
     assert S.SpMM_SplitK_API(0, 0, 0, 0, 0, 0, 128, 16, 128, 0, 2) == 1  # split-K without a workspace
+    assert S.SpMM_SplitK_API_BiasAct(0, 0, 0, 0, 0, 0, 64, 24, 64, 0, 1, 0, 0) == 999
+    assert S.SpMM_SplitK_API_BiasAct(0, 0, 0, 0, 0, 0, 64, 16, 64, 0, 1, 0, 3) == 1  # unknown activation

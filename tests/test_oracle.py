@@ -229,3 +229,46 @@ def test_splitk_reduce_and_error_metric(oracle):
     assert np.array_equal(oracle.splitk_reduce_fp16(ws, M, N, sk), want)
     a, b = ws[0], ws[1]
     assert np.isclose(oracle.total_error(a, b), np.abs(a.astype(np.float64) - b.astype(np.float64)).sum())
+
+
+# ---------------------------------------------------------------- bias + activation tail
+
+def _gelu64(x):
+    return 0.5 * x * (1.0 + np.tanh(0.7978845608028654 * (x + 0.044715 * x ** 3)))
+
+
+@pytest.mark.parametrize("act", [0, 1, 2])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_spmm_bias_act_against_float64(oracle, act, with_bias):
+    """C = fp16(act(W X + bias)) against numpy float64: a wrong sign, a bias added after the activation or along
+    the wrong axis, or ReLU/GELU swapped all fail this."""
+    from spmspm_amd.synthetic import make_activations, make_weight
+    M, K, N = 192, 256, 16
+    W = make_weight(M, K, 0.6, seed=5)
+    X = make_activations(K, N, seed=5)
+    e = oracle.encode(W, M, K)
+    vals, glo, bmp = e["values"], e["global"], e["bitmap"]
+    bias = (np.linspace(-1.5, 1.5, M)).astype(np.float16) if with_bias else None
+    got = oracle.spmm_bias_act(vals, bmp, glo, X, M, N, K, 2, bias, act).astype(np.float64)
+    pre = X.astype(np.float64) @ W.astype(np.float64).T
+    if with_bias:
+        pre = pre + bias.astype(np.float64)[None, :]
+    ref = pre if act == 0 else (np.maximum(pre, 0.0) if act == 1 else _gelu64(pre))
+    assert np.abs(got - ref).max() <= 1e-2 * np.abs(ref).max()
+    assert np.linalg.norm(got - ref) <= 2e-3 * np.linalg.norm(ref)
+    if act == 1:
+        assert (got >= 0).all() and (got[pre < -1e-2] == 0).all()
+
+
+def test_spmm_bias_act_reduces_to_plain_spmm(oracle):
+    from spmspm_amd.synthetic import make_activations, make_weight
+    M, K, N = 128, 128, 8
+    W = make_weight(M, K, 0.5, seed=6)
+    X = make_activations(K, N, seed=6)
+    e = oracle.encode(W, M, K)
+    vals, glo, bmp = e["values"], e["global"], e["bitmap"]
+    a = oracle.spmm(vals, bmp, glo, X, M, N, K, 1, False)
+    b = oracle.spmm_bias_act(vals, bmp, glo, X, M, N, K, 1, None, 0)
+    c = oracle.spmm_bias_act(vals, bmp, glo, X, M, N, K, 1, np.zeros(M, np.float16), 0)
+    assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
+    assert np.array_equal(a.view(np.uint16), c.view(np.uint16))

@@ -336,3 +336,54 @@ def test_calls_recorded_in_a_hip_graph_replay_correctly(torch, oracle):
             chain(side)  # eager work between replays
             side.synchronize()
             assert np.array_equal(got.view(np.uint16), bufs[2].cpu().numpy().view(np.uint16)), "eager != replay"
+
+
+@pytest.mark.parametrize("M,K,N,s,sk", [(256, 512, 16, 0.6, 1), (512, 1024, 8, 0.7, 4), (1024, 256, 32, 0.5, 0),
+                                        (320, 4096, 64, 0.6, 0), (128, 128, 128, 0.3, 2)])
+@pytest.mark.parametrize("act", [0, 1, 2])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_bias_activation_entry_point(torch, oracle, M, K, N, s, sk, act, with_bias):
+    """SpMM_SplitK_API_BiasAct against the oracle's fp32 tail and against float64; a garbage workspace on entry."""
+    W = make_weight(M, K, s, seed=M + N + act)
+    X = make_activations(K, N, seed=K + act)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    dev = Device(torch, comp)
+    bias = (np.random.default_rng(M).uniform(-2, 2, M)).astype(np.float16) if with_bias else None
+    b = None if bias is None else torch.from_numpy(bias.view(np.int16).copy()).to("cuda:0")
+    x = torch.from_numpy(X.view(np.int16).copy()).to("cuda:0")
+    out = torch.full((N, M), 0x7e00, dtype=torch.int16, device="cuda:0")
+    nbytes = S.SpMM_WorkspaceBytesBiasAct(M, N, K, sk)
+    assert nbytes >= 4 * M * N
+    ws = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device="cuda:0")
+    print(f"case M={M} K={K} N={N} sk={sk} act={act} bias={with_bias}", flush=True)
+    err = S.SpMM_SplitK_API_BiasAct(None, dev.values, dev.bitmaps, dev.offsets, x, out, M, N, K, ws, sk, b, act)
+    assert err == 0
+    torch.cuda.synchronize()
+    C = out.cpu().numpy().view(np.float16)
+    sk_eff = sk if sk > 0 else S.SpMM_SplitK_Auto(M, N, K)
+    ref = oracle.spmm_bias_act(comp.values, comp.bitmaps, comp.offsets, X, M, N, K, sk_eff, bias, act)
+    assert_spmm_close(C, ref, "vs oracle")
+    pre = X.astype(np.float64) @ W.astype(np.float64).T + (0 if bias is None else bias.astype(np.float64)[None, :])
+    ref64 = pre if act == 0 else (np.maximum(pre, 0) if act == 1
+                                  else 0.5 * pre * (1 + np.tanh(0.7978845608028654 * (pre + 0.044715 * pre ** 3))))
+    assert_spmm_close(C, ref64, "vs float64")
+    if act == 0 and not with_bias:  # the tail switched off is the plain entry point, bit for bit
+        assert np.array_equal(C.view(np.uint16), dev.spmm(X, sk).view(np.uint16))
+
+
+def test_bias_activation_errors_and_layer(torch, oracle, capfd):
+    t = torch.zeros(64, dtype=torch.int16, device="cuda:0")
+    assert S.SpMM_SplitK_API_BiasAct(None, t, t, t, t, t, 64, 16, 64, t, 1, None, 7) == S.api.HIP_ERROR_INVALID_VALUE
+    assert "activation" in capfd.readouterr().out
+    assert S.SpMM_SplitK_API_BiasAct(None, t, t, t, t, t, 64, 16, 64, None, 1, None, 1) == S.api.HIP_ERROR_INVALID_VALUE
+    assert "workspace" in capfd.readouterr().out
+    M, K, N = 256, 256, 16
+    W = make_weight(M, K, 0.5, seed=3)
+    X = make_activations(K, N, seed=3)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    bias = np.linspace(-1, 1, M).astype(np.float16)
+    lin = S.SparseLinear(comp, bias=bias, activation=S.ACT_RELU)
+    y = lin(torch.from_numpy(X.view(np.int16).copy()).to("cuda:0").view(torch.float16))
+    torch.cuda.synchronize()
+    ref = oracle.spmm_bias_act(comp.values, comp.bitmaps, comp.offsets, X, M, N, K, S.SpMM_SplitK_Auto(M, N, K), bias, 1)
+    assert_spmm_close(y.cpu().numpy(), ref, "layer")
