@@ -40,6 +40,7 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-dense", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    p.add_argument("--no-encoder", action="store_true", help="skip timing the device encoder on the workload's W")
     p.add_argument("--no-chain", action="store_true",
                    help="skip the OPT-13B decode-step chain (40 layers x 4 linears, sparse vs dense, same run)")
     p.add_argument("--chain-layers", type=int, default=40)
@@ -109,6 +110,28 @@ def cpu_baseline(comp, X, seconds):
         "seconds_per_pass": t, "passes": reps,
         "encoder_melems_per_s_1thread": enc_rows * K / t_enc / 1e6,
     }
+
+
+def device_encoder(torch, S, dev, W, comp, host_encode_s):
+    """Times the device encoder (both calls, incl. the read-back of the value count between them) on the
+    workload's dense W resident in HBM and checks its arrays against the host encoder's."""
+    Wd = torch.from_numpy(W.view(np.int16)).to(dev).view(torch.float16)
+    vals, bm, off = S.InitSparseMatrixA_bitmap_device(Wd)
+    torch.cuda.synchronize()
+    same = (np.array_equal(off.cpu().numpy(), comp.offsets) and np.array_equal(bm.cpu().numpy().view(np.uint64), comp.bitmaps)
+            and np.array_equal(vals.cpu().numpy().view(np.uint16), comp.values))
+    reps = 5
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        S.InitSparseMatrixA_bitmap_device(Wd)
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / reps
+    algo = 2 * W.size + 2 * comp.values.size + 8 * comp.bitmaps.size + 4 * comp.offsets.size
+    moved = algo + 2 * W.size  # W is read twice
+    return {"ms": t * 1e3, "identical_to_host_encoder": bool(same), "algorithmic_bytes": int(algo),
+            "gbs_algorithmic": algo / t / 1e9, "gbs_moved": moved / t / 1e9, "frac_of_hbm_peak": algo / t / 1e9 / HBM_PEAK_GBS,
+            "host_encoder_ms": host_encode_s * 1e3, "host_threads": os.cpu_count(),
+            "what": "dense fp16 W in HBM -> bitmaps, offsets, values in HBM; W read once = algorithmic, read twice = moved"}
 
 
 def decode_chain(torch, S, dev, layers, seed):
@@ -325,6 +348,8 @@ def main():
         "dense_fp16": dense,
         "host": {"generate_s": t_gen, "encode_s": t_enc, "encode_threads": os.cpu_count()},
     }
+    if not a.no_encoder:
+        out["device_encoder"] = device_encoder(torch, S, dev, W, comp, t_enc)
     if not a.no_chain:
         del layers, xs, outs
         torch.cuda.empty_cache()

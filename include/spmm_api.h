@@ -136,6 +136,22 @@ int InitSparseMatrixA_bitmap(uint16_t* A_h, int M, int K, int tile_M, int tile_M
                              uint64_t** bitmap, int* max_nnz_count);
 
 /*
+ * Device encoder: the same arrays as InitSparseMatrixA_bitmap, bit for bit, from a dense row-major fp16 W that
+ * already sits in device memory (no counterpart in the reference, whose only encoder is the single-threaded host
+ * function csrc/SpMM_API.cuh:112-241).  M and K must be multiples of 64 (else 1, hipErrorInvalidValue).
+ * All pointers are device memory; both calls are asynchronous on `stream`.
+ *   SpMM_EncodeDevice_Bitmaps  writes `bitmaps` (64*G uint64) and `offsets` (TileOffsets_global, G+1 ints),
+ *                              G = (M/64)*(K/64).
+ *   (the caller reads offsets[G], the number of halves `values` must hold, and allocates it)
+ *   SpMM_EncodeDevice_Values   writes `values` (compact non-zeros, every group tile's run zero-padded to a
+ *                              multiple of 8), given the `offsets` of the first call.
+ * The per-tile counts, strip offsets and max-nnz hint of the host encoder are not produced: the SpMM entry points
+ * of this library do not read them.
+ */
+int SpMM_EncodeDevice_Bitmaps(hipStream_t stream, const void* W, int M, int K, uint64_t* bitmaps, int* offsets);
+int SpMM_EncodeDevice_Values(hipStream_t stream, const void* W, int M, int K, const int* offsets, void* values);
+
+/*
  * File-to-file encoder, replaces Our_GenSparseMatrixBinFile
  * (csrc/SpMM_API.cuh:243-320; called through ctypes at
  * end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:88-102).

@@ -7,6 +7,7 @@ The functions mirror the reference's public interface for this path
 from .api import (  # noqa: F401
     CompressedMatrix,
     InitSparseMatrixA_bitmap,
+    InitSparseMatrixA_bitmap_device,
     Our_GenSparseMatrixBinFile,
     SparseLinear,
     ACT_GELU,

@@ -50,6 +50,10 @@ def library():
     L.SpMM_SplitK_API_BiasAct.argtypes = [C.c_void_p] * 6 + [C.c_int] * 3 + [C.c_void_p, C.c_int, C.c_void_p, C.c_int]
     L.SpMM_WorkspaceBytesBiasAct.restype = C.c_size_t
     L.SpMM_WorkspaceBytesBiasAct.argtypes = [C.c_int] * 4
+    L.SpMM_EncodeDevice_Bitmaps.restype = C.c_int
+    L.SpMM_EncodeDevice_Bitmaps.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    L.SpMM_EncodeDevice_Values.restype = C.c_int
+    L.SpMM_EncodeDevice_Values.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     L.InitSparseMatrixA_bitmap.restype = C.c_int
     L.InitSparseMatrixA_bitmap.argtypes = [C.c_void_p] + [C.c_int] * 8 + [
         C.POINTER(_u16p), C.POINTER(_i32p), C.POINTER(_i32p), C.POINTER(_i32p), C.POINTER(_u64p), _i32p]
@@ -206,6 +210,33 @@ def SpMM_SplitK_API(stream, values, bitmaps, offsets, X, C_out, M, N, K, workspa
 
 
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
+
+
+def InitSparseMatrixA_bitmap_device(W, stream=None):
+    """Device encoder: W is a contiguous [M][K] fp16 tensor in device memory.  Returns (values int16[offsets[G]],
+    bitmaps int64[64*G], offsets int32[G+1]) on W's device, identical to the host encoder's arrays.  Synchronises
+    once to read the number of values."""
+    import torch
+    if W.dtype != torch.float16 or W.dim() != 2 or not W.is_contiguous() or not W.is_cuda:
+        raise ValueError("W must be a contiguous [M][K] fp16 tensor on the device")
+    M, K = W.shape
+    if M % 64 or K % 64:
+        raise ValueError("M and K must be multiples of 64")
+    G = (M // 64) * (K // 64)
+    bitmaps = torch.empty(64 * G, dtype=torch.int64, device=W.device)
+    offsets = torch.empty(G + 1, dtype=torch.int32, device=W.device)
+    L = library()
+    err = L.SpMM_EncodeDevice_Bitmaps(_stream_handle(stream), _ptr(W), M, K, _ptr(bitmaps), _ptr(offsets))
+    if err != HIP_SUCCESS:
+        raise RuntimeError(f"SpMM_EncodeDevice_Bitmaps failed with hipError_t {err}")
+    if stream is not None:
+        stream.synchronize()
+    n = int(offsets[-1].item())
+    values = torch.empty(max(n, 8), dtype=torch.int16, device=W.device)
+    err = L.SpMM_EncodeDevice_Values(_stream_handle(stream), _ptr(W), M, K, _ptr(offsets), _ptr(values))
+    if err != HIP_SUCCESS:
+        raise RuntimeError(f"SpMM_EncodeDevice_Values failed with hipError_t {err}")
+    return values[:n] if n else values[:0], bitmaps, offsets
 
 
 def SpMM_WorkspaceBytesBiasAct(M, N, K, Split_K):

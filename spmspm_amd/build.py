@@ -10,7 +10,7 @@ CSRC = os.path.join(PKG, "csrc")
 LIBDIR = os.path.join(PKG, "lib")
 LIBPATH = os.path.join(LIBDIR, "libSpMM_API.so")
 
-SOURCES = ["spmm_api.hip", "encoder.cpp"]
+SOURCES = ["spmm_api.hip", "encoder_device.hip", "encoder.cpp"]
 # Packed-fp32 VALU forms are switched off for every device compile.
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared", "-fvisibility=default",

@@ -1,0 +1,256 @@
+// Device-side TCA-BME encoder for gfx950: dense fp16 W in HBM -> bitmaps, offsets, values in HBM, bit-identical
+// to the host encoder (csrc/SpMM_API.cuh:112-241 in the reference; spmspm_amd/csrc/encoder.cpp here).
+//
+// Byte work bound by HBM: W is read twice (8 KB per 64x64 group tile each time), the compressed arrays are
+// written once.  Three kernels on the caller's stream:
+//   encode_bitmaps   one wave per group tile; lane t owns 8x8 tile t (storage order 16*strip + 4*q + 2*j + i),
+//                    reads its eight 16-byte rows (the 64 lanes of one load cover eight full 128-byte lines),
+//                    builds the 64-bit mask (bit 8*r + c, non-zero test as the reference's half2float(v) != 0:
+//                    -0.0 is dropped, NaN and subnormals are kept) and the wave writes the group tile's padded
+//                    population to offsets[g + 1];
+//   scan_*           in-place running sum of offsets[1..G], offsets[0] = 0 (three small kernels, no scratch);
+//   encode_values    one wave per group tile again: a wave prefix sum of the tile populations gives every
+//                    lane the position of its first value, the lanes compact their non-zeros into LDS in
+//                    storage order, the run is padded with zeros to a multiple of eight and copied out with
+//                    16-byte stores.
+// The caller reads offsets[G] between the second and third kernel to size `values`.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+
+#include "spmm_api.h"
+
+namespace spmm_enc {
+
+constexpr int kWavesPerWG = 4;
+constexpr int kThreads    = 64 * kWavesPerWG;
+
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ int dpp_add(int x)
+{
+    return x + __builtin_amdgcn_update_dpp(0, x, kCtrl, kRowMask, 0xf, true);
+}
+
+__device__ __forceinline__ int wave_inclusive_scan(int x)
+{
+    x = dpp_add<0x111, 0xf>(x); // row_shr:1
+    x = dpp_add<0x112, 0xf>(x); // row_shr:2
+    x = dpp_add<0x114, 0xf>(x); // row_shr:4
+    x = dpp_add<0x118, 0xf>(x); // row_shr:8
+    x = dpp_add<0x142, 0xa>(x); // row_bcast:15 into rows 1 and 3
+    x = dpp_add<0x143, 0xc>(x); // row_bcast:31 into rows 2 and 3
+    return x;
+}
+
+// The lane's 8x8 tile of group tile g: eight rows of eight halves, and its bitmap.
+struct LaneTile {
+    uint4    row[8];
+    unsigned lo, hi;
+};
+
+__device__ __forceinline__ unsigned nonzero_bits(uint4 v) // bit c set when half c of the row is not +-0
+{
+    unsigned m = 0;
+    m |= (v.x & 0x00007fffu) ? 1u : 0u;
+    m |= (v.x & 0x7fff0000u) ? 2u : 0u;
+    m |= (v.y & 0x00007fffu) ? 4u : 0u;
+    m |= (v.y & 0x7fff0000u) ? 8u : 0u;
+    m |= (v.z & 0x00007fffu) ? 16u : 0u;
+    m |= (v.z & 0x7fff0000u) ? 32u : 0u;
+    m |= (v.w & 0x00007fffu) ? 64u : 0u;
+    m |= (v.w & 0x7fff0000u) ? 128u : 0u;
+    return m;
+}
+
+__device__ __forceinline__ LaneTile load_lane_tile(const uint16_t* __restrict__ W, int K, int g, int lane)
+{
+    const int nkb = K >> 6;
+    const int gm = g / nkb, gk = g - gm * nkb;
+    const int strip = lane >> 4, q = (lane >> 2) & 3, j = (lane >> 1) & 1, i = lane & 1;
+    const size_t r0 = (size_t)gm * 64 + strip * 16 + i * 8;
+    const size_t c0 = (size_t)gk * 64 + q * 16 + j * 8;
+    LaneTile     t;
+    t.lo = t.hi = 0;
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+        t.row[r] = *reinterpret_cast<const uint4*>(W + (r0 + r) * (size_t)K + c0);
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+        t.lo |= nonzero_bits(t.row[r]) << (8 * r);
+#pragma unroll
+    for (int r = 4; r < 8; ++r)
+        t.hi |= nonzero_bits(t.row[r]) << (8 * (r - 4));
+    return t;
+}
+
+__global__ __launch_bounds__(kThreads) void encode_bitmaps(const uint16_t* __restrict__ W, int K, int G,
+                                                           uint64_t* __restrict__ bitmaps, int* __restrict__ offsets)
+{
+    const int lane = threadIdx.x & 63;
+    const int g    = blockIdx.x * kWavesPerWG + (threadIdx.x >> 6);
+    if (g >= G)
+        return;
+    const LaneTile t = load_lane_tile(W, K, g, lane);
+    bitmaps[(size_t)g * 64 + lane] = ((uint64_t)t.hi << 32) | t.lo;
+    const int total = __builtin_amdgcn_readlane(wave_inclusive_scan(__builtin_popcount(t.lo) + __builtin_popcount(t.hi)), 63);
+    if (lane == 0)
+        offsets[g + 1] = (total + 7) & ~7; // the run is padded to a multiple of eight values
+}
+
+// offsets[0] = 0, offsets[1..G] <- running sum, in place and without scratch memory, in three small kernels
+// over c[i] = offsets[1 + i]:
+//   scan_blocks        every block of 1024 counts becomes its own inclusive sum (its last element = block total);
+//   scan_block_totals  one workgroup turns the blocks' last elements into global inclusive sums;
+//   add_block_prefix   block b >= 1 adds the last element of block b - 1 to all its elements but the last.
+constexpr int kScanBlock = 1024;
+
+// inclusive sum over the 256 threads of a workgroup (four waves); `red` is four ints of LDS
+__device__ __forceinline__ int workgroup_inclusive_scan_256(int x, int* red)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int       inc  = wave_inclusive_scan(x);
+    if (lane == 63)
+        red[wave] = inc;
+    __syncthreads();
+    int before = 0;
+    for (int w = 0; w < wave; ++w)
+        before += red[w];
+    __syncthreads();
+    return inc + before;
+}
+
+__global__ __launch_bounds__(256) void scan_blocks(int* __restrict__ c, int G)
+{
+    __shared__ int buf[kScanBlock];
+    __shared__ int red[4];
+    const int base = blockIdx.x * kScanBlock;
+    for (int i = threadIdx.x; i < kScanBlock; i += 256)
+        buf[i] = base + i < G ? c[base + i] : 0;
+    __syncthreads();
+    int v[4], s = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        s += buf[4 * threadIdx.x + j];
+        v[j] = s;
+    }
+    const int before = workgroup_inclusive_scan_256(s, red) - s;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        buf[4 * threadIdx.x + j] = v[j] + before;
+    __syncthreads();
+    for (int i = threadIdx.x; i < kScanBlock; i += 256)
+        if (base + i < G)
+            c[base + i] = buf[i];
+}
+
+__global__ __launch_bounds__(256) void scan_block_totals(int* __restrict__ offsets, int G)
+{
+    __shared__ int red[4];
+    int*      c  = offsets + 1;
+    const int nb = (G + kScanBlock - 1) / kScanBlock;
+    int       carry = 0;
+    if (threadIdx.x == 0)
+        offsets[0] = 0;
+    for (int b0 = 0; b0 < nb; b0 += 256) { // 256 blocks (262144 group tiles) per round
+        const int b    = b0 + threadIdx.x;
+        const int last = ((b + 1) * kScanBlock < G ? (b + 1) * kScanBlock : G) - 1;
+        const int x    = b < nb ? c[last] : 0;
+        const int inc  = workgroup_inclusive_scan_256(x, red) + carry;
+        if (b < nb)
+            c[last] = inc;
+        __shared__ int total;
+        if (threadIdx.x == 255)
+            total = inc;
+        __syncthreads();
+        carry = total;
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(256) void add_block_prefix(int* __restrict__ c, int G)
+{
+    const int b    = blockIdx.x + 1;
+    const int base = b * kScanBlock;
+    const int end  = (base + kScanBlock < G ? base + kScanBlock : G) - 1; // the last element is already global
+    const int add  = c[base - 1];
+    for (int i = base + threadIdx.x; i < end; i += 256)
+        c[i] += add;
+}
+
+__global__ __launch_bounds__(kThreads) void encode_values(const uint16_t* __restrict__ W, int K, int G,
+                                                          const int* __restrict__ offsets,
+                                                          uint16_t* __restrict__ values)
+{
+    __shared__ __attribute__((aligned(16))) uint16_t stage[kWavesPerWG][4096 + 8];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g    = blockIdx.x * kWavesPerWG + wave;
+    if (g >= G)
+        return;
+    const LaneTile t   = load_lane_tile(W, K, g, lane);
+    const int      pc  = __builtin_popcount(t.lo) + __builtin_popcount(t.hi);
+    const int      inc = wave_inclusive_scan(pc);
+    const int      total = __builtin_amdgcn_readlane(inc, 63);
+    uint16_t*      out = stage[wave];
+    int            p   = inc - pc; // position of this tile's first value in the group tile's run
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const unsigned bits = ((r < 4 ? t.lo : t.hi) >> (8 * (r & 3))) & 0xffu;
+        const unsigned d[4] = {t.row[r].x, t.row[r].y, t.row[r].z, t.row[r].w};
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            if (bits & (1u << c))
+                out[p++] = (uint16_t)(d[c >> 1] >> (16 * (c & 1)));
+    }
+    const int padded = (total + 7) & ~7;
+    if (lane < padded - total)
+        out[total + lane] = 0;
+    __builtin_amdgcn_wave_barrier(); // the wave's own LDS writes are ordered before its reads below
+    const int base = offsets[g];
+    for (int i = lane; i < (padded >> 3); i += 64)
+        reinterpret_cast<uint4*>(values + base)[i] = reinterpret_cast<const uint4*>(out)[i];
+}
+
+inline int check(int M, int K)
+{
+    if (M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0) {
+        std::printf("MM_Sparse_API Error: M (%d) and K (%d) must be positive multiples of 64!\n", M, K);
+        std::fflush(stdout);
+        return (int)hipErrorInvalidValue;
+    }
+    return 0;
+}
+
+} // namespace spmm_enc
+
+extern "C" int SpMM_EncodeDevice_Bitmaps(hipStream_t stream, const void* W, int M, int K, uint64_t* bitmaps,
+                                         int* offsets)
+{
+    if (int e = spmm_enc::check(M, K))
+        return e;
+    const int G = (M / 64) * (K / 64);
+    (void)hipGetLastError();
+    dim3 grid((unsigned)((G + spmm_enc::kWavesPerWG - 1) / spmm_enc::kWavesPerWG), 1, 1);
+    hipLaunchKernelGGL(spmm_enc::encode_bitmaps, grid, dim3(spmm_enc::kThreads, 1, 1), 0, stream,
+                       static_cast<const uint16_t*>(W), K, G, bitmaps, offsets);
+    const int nb = (G + spmm_enc::kScanBlock - 1) / spmm_enc::kScanBlock;
+    hipLaunchKernelGGL(spmm_enc::scan_blocks, dim3((unsigned)nb, 1, 1), dim3(256, 1, 1), 0, stream, offsets + 1, G);
+    hipLaunchKernelGGL(spmm_enc::scan_block_totals, dim3(1, 1, 1), dim3(256, 1, 1), 0, stream, offsets, G);
+    if (nb > 1)
+        hipLaunchKernelGGL(spmm_enc::add_block_prefix, dim3((unsigned)(nb - 1), 1, 1), dim3(256, 1, 1), 0, stream,
+                           offsets + 1, G);
+    return (int)hipGetLastError();
+}
+
+extern "C" int SpMM_EncodeDevice_Values(hipStream_t stream, const void* W, int M, int K, const int* offsets,
+                                        void* values)
+{
+    if (int e = spmm_enc::check(M, K))
+        return e;
+    const int G = (M / 64) * (K / 64);
+    (void)hipGetLastError();
+    dim3 grid((unsigned)((G + spmm_enc::kWavesPerWG - 1) / spmm_enc::kWavesPerWG), 1, 1);
+    hipLaunchKernelGGL(spmm_enc::encode_values, grid, dim3(spmm_enc::kThreads, 1, 1), 0, stream,
+                       static_cast<const uint16_t*>(W), K, G, offsets, static_cast<uint16_t*>(values));
+    return (int)hipGetLastError();
+}

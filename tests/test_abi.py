@@ -19,7 +19,8 @@ def test_header_declares_the_expected_entry_points():
     names = _declared_functions()
     for n in ("SpMM_SplitK_API", "SpMM_SplitK_API_bitmap_v3", "InitSparseMatrixA_bitmap",
               "Our_GenSparseMatrixBinFile", "SpMM_SplitK_Auto", "SpMM_WorkspaceBytes", "SpMM_Version", "SpMM_TimeNextCall",
-              "SpMM_SplitK_API_BiasAct", "SpMM_WorkspaceBytesBiasAct"):
+              "SpMM_SplitK_API_BiasAct", "SpMM_WorkspaceBytesBiasAct", "SpMM_EncodeDevice_Bitmaps",
+              "SpMM_EncodeDevice_Values"):
         assert n in names
 
 

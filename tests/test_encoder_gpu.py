@@ -1,0 +1,82 @@
+"""Device encoder (SpMM_EncodeDevice_*) against the host encoder, bit for bit, and its output fed to the SpMM."""
+import numpy as np
+import pytest
+
+import spmspm_amd as S
+from spmspm_amd.synthetic import make_activations, make_weight
+
+from conftest import assert_spmm_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+def _special_matrix(M, K, seed):
+    """Random sparse matrix sprinkled with -0.0, NaN, +-inf and subnormals, plus empty and full group tiles."""
+    rng = np.random.default_rng(seed)
+    W = make_weight(M, K, 0.6, seed=seed)
+    u = W.view(np.uint16)
+    for pat in (0x8000, 0x7e00, 0xfe01, 0x7c00, 0xfc00, 0x0001, 0x83ff):
+        idx = rng.integers(0, M * K, 50)
+        u.reshape(-1)[idx] = pat
+    W[:64, :64] = 0                                      # an empty group tile
+    W[64:128, 64:128] = np.float16(1.5)                  # a completely full one
+    u[128:192, :64] = 0x8000                             # all -0.0: encodes as empty
+    return W
+
+
+@pytest.mark.parametrize("M,K,sparsity", [(64, 64, 0.5), (128, 192, 0.7), (512, 1024, 0.9), (1024, 256, 0.0),
+                                          (256, 256, 1.0), (2048, 4096, 0.6), (65536, 64, 0.5)])
+def test_device_encoder_is_bit_identical_to_the_host_encoder(torch, M, K, sparsity):
+    W = _special_matrix(M, K, seed=M + K) if (M >= 192 and K >= 128) else make_weight(M, K, sparsity, seed=M + K)
+    if sparsity == 1.0:
+        W[:] = 0
+    comp = S.InitSparseMatrixA_bitmap(W)
+    Wd = torch.from_numpy(W.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+    print(f"case M={M} K={K} s={sparsity}", flush=True)
+    values, bitmaps, offsets = S.InitSparseMatrixA_bitmap_device(Wd)
+    torch.cuda.synchronize()
+    assert np.array_equal(offsets.cpu().numpy(), comp.offsets)
+    assert np.array_equal(bitmaps.cpu().numpy().view(np.uint64), comp.bitmaps)
+    assert np.array_equal(values.cpu().numpy().view(np.uint16), comp.values)
+
+
+def test_device_encoded_weights_multiply_correctly(torch, oracle):
+    M, K, N = 1024, 2048, 16
+    W = make_weight(M, K, 0.7, seed=77)
+    X = make_activations(K, N, seed=77)
+    Wd = torch.from_numpy(W.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+    values, bitmaps, offsets = S.InitSparseMatrixA_bitmap_device(Wd)
+    x = torch.from_numpy(X.view(np.int16).copy()).to("cuda:0")
+    out = torch.empty((N, M), dtype=torch.int16, device="cuda:0")
+    ws = torch.empty(S.SpMM_WorkspaceBytes(M, N, K, 0) + 16, dtype=torch.uint8, device="cuda:0")
+    assert S.SpMM_SplitK_API(None, values, bitmaps, offsets, x, out, M, N, K, ws, 0) == 0
+    torch.cuda.synchronize()
+    ref = X.astype(np.float64) @ W.astype(np.float64).T
+    assert_spmm_close(out.cpu().numpy().view(np.float16), ref, "device-encoded weights")
+
+
+def test_device_encoder_rejects_ragged_shapes(torch, capfd):
+    t = torch.zeros(64, dtype=torch.int16, device="cuda:0")
+    L = S.library()
+    assert L.SpMM_EncodeDevice_Bitmaps(None, t.data_ptr(), 100, 64, t.data_ptr(), t.data_ptr()) == S.api.HIP_ERROR_INVALID_VALUE
+    assert "multiples of 64" in capfd.readouterr().out
+    assert L.SpMM_EncodeDevice_Values(None, t.data_ptr(), 64, 70, t.data_ptr(), t.data_ptr()) == S.api.HIP_ERROR_INVALID_VALUE
+
+
+def test_device_encoder_offsets_scan_across_many_blocks(torch):
+    """More than 1024 group tiles, not a multiple of 1024: the in-place running sum crosses block boundaries."""
+    M, K = 64 * 37, 64 * 61  # 2257 group tiles
+    W = make_weight(M, K, 0.8, seed=9)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    Wd = torch.from_numpy(W.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+    values, bitmaps, offsets = S.InitSparseMatrixA_bitmap_device(Wd)
+    torch.cuda.synchronize()
+    assert np.array_equal(offsets.cpu().numpy(), comp.offsets)
+    assert np.array_equal(values.cpu().numpy().view(np.uint16), comp.values)
