@@ -40,6 +40,8 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-dense", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    p.add_argument("--no-qkv", action="store_true",
+                   help="skip the short extra measurement of the OPT-13B fused-QKV shape (BASELINE configs[1])")
     p.add_argument("--no-encoder", action="store_true", help="skip timing the device encoder on the workload's W")
     p.add_argument("--no-chain", action="store_true",
                    help="skip the OPT-13B decode-step chain (40 layers x 4 linears, sparse vs dense, same run)")
@@ -110,6 +112,62 @@ def cpu_baseline(comp, X, seconds):
         "seconds_per_pass": t, "passes": reps,
         "encoder_melems_per_s_1thread": enc_rows * K / t_enc / 1e6,
     }
+
+
+def quick_measure(torch, S, hip, dev, workload, steps, warmup, seed):
+    """The timing of main(), in short, for one more named workload: whole-call TFLOP/s, main-kernel GB/s and
+    roofline fraction, and the dense fp16 product of the same shape in the same run."""
+    from spmspm_amd.synthetic import WORKLOADS, make_activations, make_weight
+    w = WORKLOADS[workload]
+    M, K, N = w["M"], w["K"], w["N"]
+    W = make_weight(M, K, w["sparsity"], seed=seed, pruning=w["pruning"])
+    X = make_activations(K, N, seed=seed)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    algo = comp.algorithmic_bytes(N)
+    copies = max(2, -(-3 * LLC_BYTES // algo))
+    first = S.SparseLinear(comp, device=dev, split_k=0)
+    layers = [first] + [first.clone() for _ in range(copies - 1)]
+    x = torch.from_numpy(X.view(np.int16).copy()).to(dev).view(torch.float16)
+    out = torch.empty((N, M), dtype=torch.float16, device=dev)
+    stream = torch.cuda.current_stream()
+    L = S.library()
+    for l in layers:
+        l.workspace(N)
+    for i in range(warmup):
+        layers[i % copies](x, out=out, stream=stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        layers[i % copies](x, out=out, stream=stream)
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    events = [(hip.event(), hip.event()) for _ in range(steps)]
+    for i in range(steps):
+        L.SpMM_TimeNextCall(events[i][0], events[i][1])
+        layers[i % copies](x, out=out, stream=stream)
+    torch.cuda.synchronize()
+    kern = float(np.mean([hip.elapsed_ms(e0, e1) for e0, e1 in events])) / 1e3
+    for e0, e1 in events:
+        hip.rt.hipEventDestroy(e0), hip.rt.hipEventDestroy(e1)
+    rows = np.random.default_rng(2).choice(M, 64, replace=False)
+    got = out.cpu().numpy()[:, rows].astype(np.float64)
+    ref = X.astype(np.float64) @ W[rows].astype(np.float64).T
+    Wd = [torch.from_numpy(W.view(np.int16)).to(dev).view(torch.float16)]
+    Wd += [Wd[0].clone() for _ in range(max(2, -(-3 * LLC_BYTES // (2 * M * K))) - 1)]
+    for i in range(5):
+        torch.matmul(x, Wd[i % len(Wd)].t())
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        torch.matmul(x, Wd[i % len(Wd)].t())
+    torch.cuda.synchronize()
+    td = (time.perf_counter() - t0) / steps
+    flops = 2.0 * M * N * K
+    return {"workload": workload, "M": M, "K": K, "N": N, "sparsity": w["sparsity"], "pruning": w["pruning"],
+            "split_k": S.SpMM_SplitK_Auto(M, N, K), "tflops": flops / wall / 1e12, "us_per_call": wall * 1e6,
+            "kernel_avg_us": kern * 1e6, "gbs": algo / kern / 1e9, "roofline_frac": algo / kern / 1e9 / HBM_PEAK_GBS,
+            "algorithmic_bytes": int(algo), "dense_fp16_us": td * 1e6, "speedup_vs_dense": td / wall,
+            "rel_l2": float(np.linalg.norm(got - ref) / np.linalg.norm(ref))}
 
 
 def device_encoder(torch, S, dev, W, comp, host_encode_s):
@@ -348,6 +406,8 @@ def main():
         "dense_fp16": dense,
         "host": {"generate_s": t_gen, "encode_s": t_enc, "encode_threads": os.cpu_count()},
     }
+    if not a.no_qkv and a.workload != "opt13b_qkv":
+        out["opt13b_qkv"] = quick_measure(torch, S, hip, dev, "opt13b_qkv", max(20, a.steps // 2), a.warmup, a.seed)
     if not a.no_encoder:
         out["device_encoder"] = device_encoder(torch, S, dev, W, comp, t_enc)
     if not a.no_chain:
