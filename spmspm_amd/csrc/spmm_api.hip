@@ -25,15 +25,17 @@ int clamp_split_k(int split_k, int K)
     return split_k < 1 ? 1 : split_k;
 }
 
-// Picks the K split from a small cost model (units: group tiles processed by the busiest CU).
+// Picks the K split from a small cost model (units: group tiles processed by the busiest CU), fitted to whole-call
+// times (main kernel + reduction, back to back on one stream) of ten OPT-like shapes at Split_K 1..20, where its
+// choice is within 4 % of the best measured split:
 //   work     ceil(workgroups / 256) turns of (tiles per workgroup + a fixed start-up/epilogue cost);
-//   fill     with fewer than four workgroups per CU the waves cannot hide memory latency;
-//   partials every extra batch writes and re-reads an fp32 slab of M*N.
+//   fill     with fewer than two workgroups per CU the waves cannot hide each other's latencies;
+//   partials a split adds the reduction kernel, and every batch writes and re-reads an fp32 slab of M*N.
 int auto_split_k(int M, int N, int K)
 {
     const int    nkb  = K / 64;
     const long   base = (long)(M / 64) * spmm::column_blocks(N);
-    const double kCUs = 256.0, kStartupTiles = 3.0, kTileBytes = 3000.0;
+    const double kCUs = 256.0, kStartupTiles = 2.0, kFillWGsPerCU = 2.0, kReductionTiles = 2.0, kTileBytes = 2000.0;
     if (base <= 0 || nkb <= 0)
         return 1;
     int    best    = 1;
@@ -47,10 +49,10 @@ int auto_split_k(int M, int N, int K)
         const double tiles = (double)((nkb + sk - 1) / sk) + kStartupTiles;
         double       cost  = turns * tiles;
         const double per_cu = wgs / kCUs;
-        if (per_cu < 4.0)
-            cost *= 4.0 / (per_cu < 0.25 ? 0.25 : per_cu);
+        if (per_cu < kFillWGsPerCU)
+            cost *= kFillWGsPerCU / (per_cu < 0.25 ? 0.25 : per_cu);
         if (sk > 1)
-            cost += sk * ((double)M * N * 8.0 / kCUs) / kTileBytes;
+            cost += kReductionTiles + sk * ((double)M * N * 8.0 / kCUs) / kTileBytes;
         if (cost < best_c - 1e-9) {
             best_c = cost;
             best   = sk;
