@@ -111,3 +111,31 @@ def test_weight_file_missing_input_exits_like_reference(tmp_path):
     p = subprocess.run(["python", "-c", code], cwd=ROOT, capture_output=True, text=True)
     assert p.returncode == 255  # exit(-1)
     assert "cannot be opened" in p.stdout
+
+
+def test_cpu_reference_plumbing_config(oracle):
+    """The CPU-only configuration: W 4096x4096 N(0, 0.02) at 50 % sparsity, X 4096x16 U(-1, 1), seed 0 -- product
+    encoder == oracle encoder bit for bit, decode(encode(W)) == W, and the host SpMM on the encoded arrays agrees
+    with a float64 product on a sample of rows (the full oracle product is the GPU tests' reference)."""
+    from spmspm_amd.synthetic import WORKLOADS, make_activations, make_weight
+    w = WORKLOADS["cpu_plumbing_4096"]
+    M, K, N = w["M"], w["K"], w["N"]
+    W = make_weight(M, K, w["sparsity"], seed=0, pruning=w["pruning"])
+    X = make_activations(K, N, seed=0)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    e = oracle.encode(W, M, K)
+    assert np.array_equal(comp.values, e["values"]) and np.array_equal(comp.bitmaps, e["bitmap"])
+    assert np.array_equal(comp.offsets, e["global"]) and np.array_equal(comp.median, e["median"])
+    assert 0.49 < 1.0 - np.count_nonzero(W) / W.size < 0.51
+    back = oracle.decode(comp.values, comp.bitmaps, comp.offsets, M, K)
+    Wpos = W.copy()
+    Wpos[Wpos == 0] = 0  # -0.0 is not stored and comes back as +0.0
+    assert np.array_equal(back.view(np.uint16), Wpos.view(np.uint16))
+    # host SpMM on the first four row blocks only (keeps the CPU suite short)
+    rows = 256
+    g1 = (rows // 64) * (K // 64)
+    off = comp.offsets[:g1 + 1]
+    C = oracle.spmm(comp.values[:int(off[-1])], comp.bitmaps[:g1 * 64], off, X, rows, N, K, 1, False).astype(np.float64)
+    ref = X.astype(np.float64) @ W[:rows].astype(np.float64).T
+    assert np.abs(C - ref).max() <= 1e-2 * np.abs(ref).max()
+    assert np.linalg.norm(C - ref) <= 1e-3 * np.linalg.norm(ref)
