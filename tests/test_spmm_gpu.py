@@ -387,3 +387,25 @@ def test_bias_activation_errors_and_layer(torch, oracle, capfd):
     torch.cuda.synchronize()
     ref = oracle.spmm_bias_act(comp.values, comp.bitmaps, comp.offsets, X, M, N, K, S.SpMM_SplitK_Auto(M, N, K), bias, 1)
     assert_spmm_close(y.cpu().numpy(), ref, "layer")
+
+
+def test_seeded_random_shapes(torch, oracle):
+    """Forty seeded random cases (shape, columns, density incl. nearly empty and nearly full, split) through both
+    entry points against the oracle."""
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        M = 64 * int(rng.integers(1, 9))
+        K = 64 * int(rng.integers(1, 25))
+        N = int(rng.choice([8, 16, 32, 64, 128]))
+        s = float(rng.choice([0.0, 0.05, 0.3, 0.5, 0.7, 0.9, 0.99]))
+        sk = int(rng.integers(0, min(8, K // 64) + 1))
+        W = make_weight(M, K, s, seed=1000 + case)
+        X = make_activations(K, N, seed=2000 + case)
+        comp = S.InitSparseMatrixA_bitmap(W)
+        dev = Device(torch, comp)
+        print(f"case {case}: M={M} K={K} N={N} s={s} sk={sk}", flush=True)
+        sk_eff = sk if sk > 0 else S.SpMM_SplitK_Auto(M, N, K)
+        sk_eff = min(sk_eff, K // 64)
+        assert_spmm_close(dev.spmm(X, sk), _oracle_C(oracle, comp, X, sk_eff), f"case {case} api")
+        if sk > 0:
+            assert_spmm_close(dev.spmm(X, sk, "v3"), _oracle_C(oracle, comp, X, sk_eff, True), f"case {case} v3")
