@@ -44,5 +44,26 @@ def build_library(verbose=False, extra_flags=()):
     return LIBPATH
 
 
+HARNESS_SRC = os.path.join(ROOT, "tests", "cpp", "harness.cpp")
+HARNESS_PATH = os.path.join(LIBDIR, "spmm_harness")
+
+
+def build_harness(verbose=False):
+    """Compile the C++ caller (tests/cpp/harness.cpp) against the library: the reference harness's call sequence
+    through the `__half*` encoder overload and the 14-argument entry point.  Run by the GPU tests."""
+    cmd = [hipcc(), "-O2", "-std=c++17", "--offload-arch=gfx950", "-Wno-unused-command-line-argument",
+           "-I", os.path.join(ROOT, "include"), HARNESS_SRC, "-L", LIBDIR, "-lSpMM_API",
+           "-Wl,-rpath,$ORIGIN", "-o", HARNESS_PATH + ".tmp"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        sys.stderr.write(proc.stdout + proc.stderr)
+        raise RuntimeError("hipcc failed building the C++ harness")
+    os.replace(HARNESS_PATH + ".tmp", HARNESS_PATH)
+    return HARNESS_PATH
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_harness(verbose=True))

@@ -1,4 +1,6 @@
 """Parity of the HIP SpMM (through the C ABI) with the CPU oracle, the golden vectors and float64 mathematics."""
+import os
+
 import numpy as np
 import pytest
 
@@ -409,3 +411,18 @@ def test_seeded_random_shapes(torch, oracle):
         assert_spmm_close(dev.spmm(X, sk), _oracle_C(oracle, comp, X, sk_eff), f"case {case} api")
         if sk > 0:
             assert_spmm_close(dev.spmm(X, sk, "v3"), _oracle_C(oracle, comp, X, sk_eff, True), f"case {case} v3")
+
+
+@pytest.mark.parametrize("args", [(1024, 1024, 16, 70, 2), (2048, 512, 8, 50, 1), (512, 4096, 32, 60, 4),
+                                  (1024, 2048, 64, 40, 3), (256, 1024, 128, 90, 2)])
+def test_cpp_caller_of_the_library(args):
+    """tests/cpp/harness.cpp, built against libSpMM_API.so by build(): the reference harness's call sequence from
+    C++ (encoder overload with the reference's signature, 14-argument SpMM on the null stream, then the shorter
+    entry point), checked inside the program against a float64 product of sampled rows."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(S.library_path()), "spmm_harness")
+    assert os.path.exists(exe), "build it with __graft_entry__.build()"
+    print("harness", args, flush=True)
+    p = subprocess.run([exe] + [str(a) for a in args], capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0, p.stdout + p.stderr
+    assert "PASS" in p.stdout and "spmm-gfx950" in p.stdout
