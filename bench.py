@@ -106,11 +106,17 @@ def cpu_baseline(comp, X, seconds):
     t0 = time.perf_counter()
     O.encode(Wenc, enc_rows, K)
     t_enc = time.perf_counter() - t0
+    ref_rate = None
+    if O.ref_lib() is not None:  # the reference's own encoder, compiled from its source where that tree was present
+        t0 = time.perf_counter()
+        O.ref_encode(Wenc, enc_rows, K)
+        ref_rate = enc_rows * K / (time.perf_counter() - t0) / 1e6
     return {
         "value": flops / t / 1e12, "unit": "TFLOP/s", "cores": O.num_threads(), "kind": "port",
         "sample": f"rows 0..{rows} of {M} (K={K}, N={N}), {reps} passes of {t:.3f} s, host decode+GEMM, OpenMP",
         "seconds_per_pass": t, "passes": reps,
         "encoder_melems_per_s_1thread": enc_rows * K / t_enc / 1e6,
+        "reference_encoder_melems_per_s_1thread": ref_rate,
     }
 
 
