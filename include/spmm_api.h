@@ -91,6 +91,24 @@ int SpMM_SplitK_API_bitmap_v3(hipStream_t stream, const void* A, const void* Com
  */
 int SpMM_SplitK_Auto(int M, int N, int K);
 
+/*
+ * Measured Split_K choices, which SpMM_SplitK_Auto (and every call with Split_K <= 0) prefers to its built-in
+ * cost model.  They take the place of the hand-kept tables of the reference: SplitKDict
+ * (end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:23, keyed by M alone) and the SPLIT_K array of
+ * kernel_benchmark/run_all_main.sh:5.  The table is keyed by (M, N, K) and shared by all threads of the process.
+ *   TableSet    records one choice; returns 0, or hipErrorInvalidValue for a shape the library does not run.
+ *   TableLoad   adds the entries of a text file of "M N K Split_K" lines ('#' starts a comment); returns their
+ *               number, -1 if the file cannot be opened, -2 on a malformed line.
+ *   TableSave   writes the table in that format; returns the number of entries, -1 if the file cannot be written.
+ *   TableClear  empties the table.
+ * A file named by SPMM_SPLITK_TABLE in the environment is loaded the first time a choice is needed.
+ * A workspace must be sized (SpMM_WorkspaceBytes) after the table is in its final state.
+ */
+int  SpMM_SplitK_TableSet(int M, int N, int K, int Split_K);
+int  SpMM_SplitK_TableLoad(const char* path);
+int  SpMM_SplitK_TableSave(const char* path);
+void SpMM_SplitK_TableClear(void);
+
 /* Bytes of workspace SpMM_SplitK_API needs for this call (0 for Split_K == 1).
  * Split_K <= 0 means the library's own choice and returns a size that covers
  * whatever way it may split the work. */

@@ -18,6 +18,10 @@ from .api import (  # noqa: F401
     SpMM_WorkspaceBytesBiasAct,
     SpMM_SplitK_API_bitmap_v3,
     SpMM_SplitK_Auto,
+    SpMM_SplitK_TableClear,
+    SpMM_SplitK_TableLoad,
+    SpMM_SplitK_TableSave,
+    SpMM_SplitK_TableSet,
     SpMM_WorkspaceBytes,
     library,
     library_path,

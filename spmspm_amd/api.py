@@ -44,6 +44,14 @@ def library():
     L.SpMM_SplitK_API_bitmap_v3.argtypes = [C.c_void_p] * 9 + [C.c_int] * 3 + [C.c_void_p, C.c_int]
     L.SpMM_SplitK_Auto.restype = C.c_int
     L.SpMM_SplitK_Auto.argtypes = [C.c_int] * 3
+    L.SpMM_SplitK_TableSet.restype = C.c_int
+    L.SpMM_SplitK_TableSet.argtypes = [C.c_int] * 4
+    L.SpMM_SplitK_TableLoad.restype = C.c_int
+    L.SpMM_SplitK_TableLoad.argtypes = [C.c_char_p]
+    L.SpMM_SplitK_TableSave.restype = C.c_int
+    L.SpMM_SplitK_TableSave.argtypes = [C.c_char_p]
+    L.SpMM_SplitK_TableClear.restype = None
+    L.SpMM_SplitK_TableClear.argtypes = []
     L.SpMM_WorkspaceBytes.restype = C.c_size_t
     L.SpMM_WorkspaceBytes.argtypes = [C.c_int] * 4
     L.SpMM_SplitK_API_BiasAct.restype = C.c_int
@@ -180,6 +188,32 @@ def _popcount64(a):
 
 def SpMM_SplitK_Auto(M, N, K):
     return library().SpMM_SplitK_Auto(M, N, K)
+
+
+def SpMM_SplitK_TableSet(M, N, K, Split_K):
+    """Record a measured Split_K for a shape; calls with Split_K <= 0 use it instead of the cost model."""
+    rc = library().SpMM_SplitK_TableSet(M, N, K, Split_K)
+    if rc != 0:
+        raise ValueError(f"SpMM_SplitK_TableSet({M}, {N}, {K}, {Split_K}) -> {rc}")
+
+
+def SpMM_SplitK_TableLoad(path):
+    """Add the "M N K Split_K" lines of a text file to the table; returns how many were read."""
+    n = library().SpMM_SplitK_TableLoad(os.fsencode(path))
+    if n < 0:
+        raise OSError(f"{path}: " + ("cannot be opened" if n == -1 else "malformed line"))
+    return n
+
+
+def SpMM_SplitK_TableSave(path):
+    n = library().SpMM_SplitK_TableSave(os.fsencode(path))
+    if n < 0:
+        raise OSError(f"{path}: cannot be written")
+    return n
+
+
+def SpMM_SplitK_TableClear():
+    library().SpMM_SplitK_TableClear()
 
 
 def SpMM_WorkspaceBytes(M, N, K, Split_K):

@@ -5,6 +5,9 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <map>
+#include <mutex>
+#include <tuple>
 
 #include "spmm_api.h"
 #include "spmm_kernels.hiph"
@@ -61,6 +64,70 @@ int auto_split_k(int M, int N, int K)
     return best;
 }
 
+// Measured choices that take precedence over the cost model (the role of the reference's SplitKDict,
+// end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:23, and of the SPLIT_K array of
+// kernel_benchmark/run_all_main.sh:5): a table keyed by (M, N, K), filled by SpMM_SplitK_TableSet or from a text
+// file of "M N K Split_K" lines.  SPMM_SPLITK_TABLE in the environment names a file that is loaded on first use.
+struct SplitTable {
+    std::mutex                                  lock;
+    std::map<std::tuple<int, int, int>, int>    entries;
+    bool                                        env_checked = false;
+};
+SplitTable& split_table()
+{
+    static SplitTable t;
+    return t;
+}
+
+// returns the number of entries read, or -1 when the file cannot be opened, -2 on a malformed line
+int load_split_table_locked(SplitTable& t, const char* path)
+{
+    std::FILE* f = std::fopen(path, "r");
+    if (!f)
+        return -1;
+    char line[256];
+    int  n = 0;
+    while (std::fgets(line, sizeof line, f)) {
+        const char* p = line;
+        while (*p == ' ' || *p == '\t')
+            ++p;
+        if (*p == '#' || *p == '\n' || *p == '\r' || *p == 0)
+            continue;
+        int m, nn, k, sk;
+        if (std::sscanf(p, "%d %d %d %d", &m, &nn, &k, &sk) != 4 || m <= 0 || nn <= 0 || k <= 0 || sk < 1) {
+            std::fclose(f);
+            return -2;
+        }
+        t.entries[std::make_tuple(m, nn, k)] = sk;
+        ++n;
+    }
+    std::fclose(f);
+    return n;
+}
+
+int split_k_for(int M, int N, int K)
+{
+    SplitTable& t = split_table();
+    {
+        std::lock_guard<std::mutex> g(t.lock);
+        if (!t.env_checked) {
+            t.env_checked = true;
+            if (const char* e = std::getenv("SPMM_SPLITK_TABLE")) {
+                const int n = load_split_table_locked(t, e);
+                if (n < 0) {
+                    std::printf("MM_Sparse_API Warning: SPMM_SPLITK_TABLE=%s %s; using the built-in choice.\n", e,
+                                n == -1 ? "cannot be opened" : "has a malformed line");
+                    std::fflush(stdout);
+                }
+            }
+        }
+        auto it = t.entries.find(std::make_tuple(M, N, K));
+        if (it != t.entries.end())
+            return clamp_split_k(it->second, K);
+    }
+    return clamp_split_k(auto_split_k(M, N, K), K);
+}
+
 int check_shape(int M, int N, int K)
 {
     if (!supported_n(N)) {
@@ -110,14 +177,56 @@ extern "C" int SpMM_SplitK_Auto(int M, int N, int K)
 {
     if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
         return 1;
-    return clamp_split_k(auto_split_k(M, N, K), K);
+    return split_k_for(M, N, K);
+}
+
+extern "C" int SpMM_SplitK_TableSet(int M, int N, int K, int Split_K)
+{
+    if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0 || Split_K < 1)
+        return (int)hipErrorInvalidValue;
+    SplitTable&                 t = split_table();
+    std::lock_guard<std::mutex> g(t.lock);
+    t.entries[std::make_tuple(M, N, K)] = Split_K;
+    return 0;
+}
+
+extern "C" int SpMM_SplitK_TableLoad(const char* path)
+{
+    if (path == nullptr)
+        return -1;
+    SplitTable&                 t = split_table();
+    std::lock_guard<std::mutex> g(t.lock);
+    return load_split_table_locked(t, path);
+}
+
+extern "C" int SpMM_SplitK_TableSave(const char* path)
+{
+    if (path == nullptr)
+        return -1;
+    SplitTable&                 t = split_table();
+    std::lock_guard<std::mutex> g(t.lock);
+    std::FILE*                  f = std::fopen(path, "w");
+    if (!f)
+        return -1;
+    std::fprintf(f, "# M N K Split_K\n");
+    for (const auto& e : t.entries)
+        std::fprintf(f, "%d %d %d %d\n", std::get<0>(e.first), std::get<1>(e.first), std::get<2>(e.first), e.second);
+    std::fclose(f);
+    return (int)t.entries.size();
+}
+
+extern "C" void SpMM_SplitK_TableClear(void)
+{
+    SplitTable&                 t = split_table();
+    std::lock_guard<std::mutex> g(t.lock);
+    t.entries.clear();
 }
 
 extern "C" size_t SpMM_WorkspaceBytes(int M, int N, int K, int Split_K)
 {
     if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
         return 0;
-    int sk = clamp_split_k(Split_K <= 0 ? auto_split_k(M, N, K) : Split_K, K);
+    int sk = Split_K <= 0 ? split_k_for(M, N, K) : clamp_split_k(Split_K, K);
     if (sk <= 1)
         return 0;
     return sizeof(float) * (size_t)M * (size_t)N * (size_t)sk;
@@ -136,7 +245,7 @@ extern "C" size_t SpMM_WorkspaceBytesBiasAct(int M, int N, int K, int Split_K)
 {
     if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
         return 0;
-    int sk = clamp_split_k(Split_K <= 0 ? auto_split_k(M, N, K) : Split_K, K);
+    int sk = Split_K <= 0 ? split_k_for(M, N, K) : clamp_split_k(Split_K, K);
     return sizeof(float) * (size_t)M * (size_t)N * (size_t)sk; // one fp32 slab even for an unsplit K
 }
 

@@ -20,7 +20,8 @@ def test_header_declares_the_expected_entry_points():
     for n in ("SpMM_SplitK_API", "SpMM_SplitK_API_bitmap_v3", "InitSparseMatrixA_bitmap",
               "Our_GenSparseMatrixBinFile", "SpMM_SplitK_Auto", "SpMM_WorkspaceBytes", "SpMM_Version", "SpMM_TimeNextCall",
               "SpMM_SplitK_API_BiasAct", "SpMM_WorkspaceBytesBiasAct", "SpMM_EncodeDevice_Bitmaps",
-              "SpMM_EncodeDevice_Values"):
+              "SpMM_EncodeDevice_Values", "SpMM_SplitK_TableSet", "SpMM_SplitK_TableLoad", "SpMM_SplitK_TableSave",
+              "SpMM_SplitK_TableClear"):
         assert n in names
 
 
@@ -54,3 +55,60 @@ def test_shape_errors_are_reported_without_a_gpu(capfd):
     assert S.SpMM_SplitK_API(0, 0, 0, 0, 0, 0, 128, 16, 128, 0, 2) == 1  # split-K without a workspace
     assert S.SpMM_SplitK_API_BiasAct(0, 0, 0, 0, 0, 0, 64, 24, 64, 0, 1, 0, 0) == 999
     assert S.SpMM_SplitK_API_BiasAct(0, 0, 0, 0, 0, 0, 64, 16, 64, 0, 1, 0, 3) == 1  # unknown activation
+
+
+def test_split_table_overrides_the_cost_model_and_round_trips_through_a_file(tmp_path):
+    import pytest
+    S.SpMM_SplitK_TableClear()
+    model, model_n32 = S.SpMM_SplitK_Auto(28672, 16, 7168), S.SpMM_SplitK_Auto(28672, 32, 7168)
+    other = model + 1
+    try:
+        S.SpMM_SplitK_TableSet(28672, 16, 7168, other)
+        S.SpMM_SplitK_TableSet(5120, 16, 5120, 1000)  # more batches than group-tile columns: clamped when used
+        assert S.SpMM_SplitK_Auto(28672, 16, 7168) == other
+        assert S.SpMM_SplitK_Auto(5120, 16, 5120) == 5120 // 64
+        assert S.SpMM_SplitK_Auto(28672, 32, 7168) == model_n32  # other N: not in the table
+        assert S.SpMM_WorkspaceBytes(28672, 16, 7168, 0) == 4 * 28672 * 16 * other
+        assert S.SpMM_WorkspaceBytesBiasAct(28672, 16, 7168, 0) == 4 * 28672 * 16 * other
+        path = tmp_path / "splitk.txt"
+        assert S.SpMM_SplitK_TableSave(path) == 2
+        lines = [l for l in path.read_text().splitlines() if not l.startswith("#")]
+        assert sorted(lines) == sorted(["28672 16 7168 %d" % other, "5120 16 5120 1000"])
+        S.SpMM_SplitK_TableClear()
+        assert S.SpMM_SplitK_Auto(28672, 16, 7168) == model
+        path.write_text("# tuned on some day\n\n  28672 16 7168 %d\n4096 16 4096 2 trailing words are ignored\n" % other)
+        assert S.SpMM_SplitK_TableLoad(path) == 2
+        assert S.SpMM_SplitK_Auto(28672, 16, 7168) == other and S.SpMM_SplitK_Auto(4096, 16, 4096) == 2
+        bad = tmp_path / "bad.txt"
+        bad.write_text("28672 16 7168\n")
+        with pytest.raises(OSError):
+            S.SpMM_SplitK_TableLoad(bad)
+        with pytest.raises(OSError):
+            S.SpMM_SplitK_TableLoad(tmp_path / "missing.txt")
+        with pytest.raises(ValueError):
+            S.SpMM_SplitK_TableSet(100, 16, 64, 2)  # not a shape the library runs
+        with pytest.raises(ValueError):
+            S.SpMM_SplitK_TableSet(128, 16, 128, 0)
+    finally:
+        S.SpMM_SplitK_TableClear()
+
+
+def test_split_table_file_named_in_the_environment_is_loaded_on_first_use(tmp_path):
+    import subprocess
+    import sys
+    path = tmp_path / "t.txt"
+    path.write_text("28672 16 7168 7\n")
+    code = "import spmspm_amd as S; print(S.SpMM_SplitK_Auto(28672, 16, 7168), S.SpMM_SplitK_Auto(4096, 16, 4096))"
+    env = dict(os.environ, SPMM_SPLITK_TABLE=str(path), PYTHONPATH=ROOT)
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True).stdout.split()
+    assert out[0] == "7" and int(out[1]) >= 1
+    env["SPMM_SPLITK_TABLE"] = str(tmp_path / "missing.txt")
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True)
+    assert "cannot be opened" in r.stdout and int(r.stdout.split()[-2]) >= 1
+
+
+def test_tuner_candidates_and_presets():
+    from spmspm_amd import tuner
+    assert tuner.candidate_splits(5120) == list(range(1, 13))
+    assert tuner.candidate_splits(256) == [1] and tuner.candidate_splits(512) == [1, 2]
+    assert (28672, 7168) in tuner.PRESETS["opt30b"] and len(tuner.PRESETS["opt13b"]) == 4

@@ -426,3 +426,31 @@ def test_cpp_caller_of_the_library(args):
     p = subprocess.run([exe] + [str(a) for a in args], capture_output=True, text=True, timeout=120)
     assert p.returncode == 0, p.stdout + p.stderr
     assert "PASS" in p.stdout and "spmm-gfx950" in p.stdout
+
+
+def test_tuner_records_a_measured_split_that_the_library_then_uses(torch, oracle, tmp_path):
+    from spmspm_amd import tuner
+    M, K, N, s = 2048, 4096, 16, 0.6
+    S.SpMM_SplitK_TableClear()
+    try:
+        res = tuner.tune([(M, K)], N, sparsity=s, iters=10, candidates=[1, 2, 4, 8])
+        best, times = res[(M, N, K)]
+        assert best in (1, 2, 4, 8) and set(times) == {1, 2, 4, 8} and all(t > 0 for t in times.values())
+        assert S.SpMM_SplitK_Auto(M, N, K) == best
+        path = tmp_path / "splitk.txt"
+        assert S.SpMM_SplitK_TableSave(path) == 1
+        # a split that only the table can have chosen, and results that do not depend on it
+        S.SpMM_SplitK_TableSet(M, N, K, 7)
+        W, X = make_weight(M, K, s, seed=21), make_activations(K, N, seed=21)
+        comp = S.InitSparseMatrixA_bitmap(W)
+        x = torch.from_numpy(X.view(np.int16).copy()).cuda().view(torch.float16)
+        layer = S.SparseLinear(comp)  # split_k=0: the library's choice, i.e. the table's
+        assert layer.workspace(N).numel() == 4 * M * N * 7
+        got = layer(x)
+        torch.cuda.synchronize()
+        want = oracle.spmm(comp.values, comp.bitmaps, comp.offsets, X, M, N, K, 7, False)
+        assert_spmm_close(got.cpu().numpy(), want)
+        S.SpMM_SplitK_TableClear()
+        assert S.SpMM_SplitK_TableLoad(path) == 1 and S.SpMM_SplitK_Auto(M, N, K) == best
+    finally:
+        S.SpMM_SplitK_TableClear()
