@@ -30,8 +30,8 @@ LLC_BYTES = 256 << 20
 def parse():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    p.add_argument("--steps", type=int, default=200)
-    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--steps", type=int, default=2000)  # 2000 x ~45 us: long enough that the start-up of the timed region (about 1 ms) does not weigh on it
+    p.add_argument("--warmup", type=int, default=100)
     p.add_argument("--workload", default="opt30b_ffn1")
     p.add_argument("--n", type=int, default=None, help="override the workload's N")
     p.add_argument("--sparsity", type=float, default=None, help="override the workload's sparsity (0..1)")
