@@ -32,7 +32,7 @@ def candidate_splits(K, limit=12):
     return [s for s in range(1, limit + 1) if s <= max(1, nkb // 4)]
 
 
-def time_split_k(layers, x, split_k, iters=40, warmup=5):
+def time_split_k(layers, x, split_k, iters=300, warmup=20):
     """Average time in microseconds of one call at this Split_K, rotating among `layers` (resident copies)."""
     import torch
     for L in layers:
@@ -50,7 +50,7 @@ def time_split_k(layers, x, split_k, iters=40, warmup=5):
     return e0.elapsed_time(e1) * 1e3 / iters
 
 
-def tune_shape(M, N, K, sparsity=0.6, candidates=None, device="cuda:0", iters=40, copies_bytes=768 << 20, seed=0):
+def tune_shape(M, N, K, sparsity=0.6, candidates=None, device="cuda:0", iters=300, copies_bytes=768 << 20, seed=0):
     """Times every candidate Split_K for one shape; returns (best_split, {split: microseconds}).
 
     The matrix is synthetic (Bernoulli mask at `sparsity`): the choice depends on the shape and on the bytes
@@ -98,7 +98,7 @@ def main(argv=None):
     ap.add_argument("--shape", action="append", default=[], metavar="MxK", help="extra shape, e.g. 28672x7168")
     ap.add_argument("--n", type=int, action="append", help="batch columns (repeatable; default 16)")
     ap.add_argument("--sparsity", type=float, default=0.6)
-    ap.add_argument("--iters", type=int, default=40)
+    ap.add_argument("--iters", type=int, default=300)
     ap.add_argument("--out", help="write the table here (text, one 'M N K Split_K' per line)")
     ap.add_argument("--json", help="also write every measured time here")
     a = ap.parse_args(argv)
