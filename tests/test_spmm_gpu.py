@@ -272,6 +272,51 @@ def test_target_shape_against_oracle(torch, oracle):
     assert_spmm_close(dev.spmm(X, 4, "v3"), want, "target v3 sk=4")
 
 
+@pytest.mark.parametrize("sparsity", [0.4, 0.5])
+def test_opt30b_ffn1_full_size_other_batches_and_sparsities(torch, sparsity):
+    """OPT-30B FFN1 28672x7168 at the denser settings of the benchmark set, N = 8 and 32, magnitude pruning:
+    sampled rows against float64 through both entry points."""
+    M, K = 28672, 7168
+    W = make_weight(M, K, sparsity, seed=7, pruning="magnitude")
+    comp = S.InitSparseMatrixA_bitmap(W)
+    dev = Device(torch, comp)
+    rng = np.random.default_rng(9)
+    rows = rng.choice(M, 96, replace=False)
+    Wrows = W[rows].astype(np.float64)
+    del W
+    for N in (8, 32):
+        X = make_activations(K, N, seed=N)
+        ref = X.astype(np.float64) @ Wrows.T
+        assert_spmm_close(dev.spmm(X, 0)[:, rows], ref, f"s={sparsity} N={N} auto")
+        assert_spmm_close(dev.spmm(X, 2, "v3")[:, rows], ref, f"s={sparsity} N={N} v3 sk=2")
+
+
+def test_opt66b_ffn2_full_size_wide_batches(torch):
+    """OPT-66B FFN2 9216x36864 at 40 % sparsity, N = 64 and 128 (the widest configuration of the benchmark set):
+    sampled rows against float64, and the sum over all rows of every output column against the same sum taken
+    on the weights first (sum_m C[n][m] = sum_k X[n][k] * sum_m W[m][k])."""
+    M, K = 9216, 36864
+    W = make_weight(M, K, 0.4, seed=3)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    dev = Device(torch, comp)
+    rng = np.random.default_rng(5)
+    rows = rng.choice(M, 48, replace=False)
+    Wrows = W[rows].astype(np.float64)
+    colsum = np.zeros(K, np.float64)
+    for r0 in range(0, M, 1024):  # in slices: a float64 copy of W would be 2.7 GB
+        colsum += W[r0:r0 + 1024].astype(np.float32).sum(axis=0, dtype=np.float64)
+    del W
+    for N in (64, 128):
+        X = (rng.integers(-8, 9, (N, K)) / 16).astype(np.float16)
+        for sk in (0, 3):
+            C = dev.spmm(X, sk)
+            assert_spmm_close(C[:, rows], X.astype(np.float64) @ Wrows.T, f"N={N} sk={sk} sampled rows")
+            got, want = C.astype(np.float64).sum(axis=1), X.astype(np.float64) @ colsum
+            # every output carries its own fp16 rounding (2^-11 relative); M of them add up in quadrature
+            tol = 4.0 * 2.0 ** -11 * np.sqrt((C.astype(np.float64) ** 2).sum(axis=1)) + 1e-6
+            assert (np.abs(got - want) <= tol).all(), f"N={N} sk={sk}: column sums off by {np.abs(got - want).max():.3e}"
+
+
 def test_error_returns_on_device(torch, capfd):
     t = torch.zeros(16, dtype=torch.int16, device="cuda:0")
     assert S.SpMM_SplitK_API(None, t, t, t, t, t, 64, 48, 64, None, 1) == S.api.HIP_ERROR_UNKNOWN
