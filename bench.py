@@ -281,8 +281,8 @@ def decode_chain(torch, S, dev, layers, seed):
 def main():
     a = parse()
     if a.gpus != 1:
-        print("bench.py: this build drives one GPU; run with --gpus 1 (the path shards by rows with no "
-              "exchange, see DESIGN.md)", file=sys.stderr)
+        print("bench.py: this build drives one GPU; run with --gpus 1 (row blocks are independent, so the path "
+              "would shard by rows without any exchange, but no multi-GPU launch is part of this build)", file=sys.stderr)
         sys.exit(2)
     import torch
 
