@@ -131,6 +131,22 @@ int SpMM_SplitK_API_BiasAct(hipStream_t stream, const void* values, const uint64
 size_t SpMM_WorkspaceBytesBiasAct(int M, int N, int K, int Split_K);
 
 /*
+ * SpMM_SplitK_API without a workspace argument and without any allocation.  It has no counterpart in the
+ * reference; it is for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  The fp32 partial sums of a split K go to a device array of
+ * SPMM_NOALLOC_SCRATCH_BYTES that the library itself holds on every GPU it runs on until the process ends.
+ * Arguments, Split_K <= 0 and results are those of SpMM_SplitK_API (the same kernels run); a call whose partial
+ * sums (4*M*N*Split_K bytes for Split_K > 1) exceed the array prints a message and returns 1
+ * (hipErrorInvalidValue) without launching anything.  The call makes no hipMalloc/hipFree; the first call on a
+ * device looks up the array's device address once (make that call outside a graph capture).
+ * All calls on one GPU share the array: calls that overlap in time on one GPU (different streams, or graphs
+ * replayed concurrently) race on it and must be serialised by the caller.
+ */
+#define SPMM_NOALLOC_SCRATCH_BYTES (32u << 20)
+int SpMM_SplitK_API_NoAlloc(hipStream_t stream, const void* values, const uint64_t* bitmaps, const int* offsets,
+                            const void* X, void* C, int M, int N, int K, int Split_K);
+
+/*
  * Host encoder, C twin of InitSparseMatrixA_bitmap
  * (csrc/SpMM_API.cuh:112-241): dense row-major fp16 W -> TCA-BME arrays.
  * Output is bit-identical to the reference's.  The tile-size arguments are

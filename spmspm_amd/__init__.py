@@ -13,7 +13,9 @@ from .api import (  # noqa: F401
     ACT_GELU,
     ACT_NONE,
     ACT_RELU,
+    NOALLOC_SCRATCH_BYTES,
     SpMM_SplitK_API,
+    SpMM_SplitK_API_NoAlloc,
     SpMM_SplitK_API_BiasAct,
     SpMM_WorkspaceBytesBiasAct,
     SpMM_SplitK_API_bitmap_v3,

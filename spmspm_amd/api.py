@@ -52,6 +52,8 @@ def library():
     L.SpMM_SplitK_TableSave.argtypes = [C.c_char_p]
     L.SpMM_SplitK_TableClear.restype = None
     L.SpMM_SplitK_TableClear.argtypes = []
+    L.SpMM_SplitK_API_NoAlloc.restype = C.c_int
+    L.SpMM_SplitK_API_NoAlloc.argtypes = [C.c_void_p] * 6 + [C.c_int] * 4
     L.SpMM_WorkspaceBytes.restype = C.c_size_t
     L.SpMM_WorkspaceBytes.argtypes = [C.c_int] * 4
     L.SpMM_SplitK_API_BiasAct.restype = C.c_int
@@ -241,6 +243,16 @@ def SpMM_SplitK_API(stream, values, bitmaps, offsets, X, C_out, M, N, K, workspa
     """C = W*X on the device (include/spmm_api.h).  Tensors or raw device addresses.  Returns the hipError_t."""
     return library().SpMM_SplitK_API(_stream_handle(stream), _ptr(values), _ptr(bitmaps), _ptr(offsets), _ptr(X),
                                      _ptr(C_out), M, N, K, _ptr(workspace), Split_K)
+
+
+NOALLOC_SCRATCH_BYTES = 32 << 20  # SPMM_NOALLOC_SCRATCH_BYTES of include/spmm_api.h
+
+
+def SpMM_SplitK_API_NoAlloc(stream, values, bitmaps, offsets, X, C_out, M, N, K, Split_K):
+    """SpMM_SplitK_API whose split-K partial sums live in the library's own device array: no workspace argument,
+    no allocation (include/spmm_api.h).  Returns the hipError_t."""
+    return library().SpMM_SplitK_API_NoAlloc(_stream_handle(stream), _ptr(values), _ptr(bitmaps), _ptr(offsets),
+                                             _ptr(X), _ptr(C_out), M, N, K, Split_K)
 
 
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2

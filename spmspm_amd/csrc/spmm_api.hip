@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <map>
@@ -280,6 +281,77 @@ extern "C" int SpMM_SplitK_API_bitmap_v3(hipStream_t stream, const void* /*A*/, 
     }
     return run(stream, Compressed_A, bitmap, TileOffsets, B, C, M_Global, N_Global, K_Global, Reduction_Workspace,
                Split_K, /*fp32_partials=*/false);
+}
+
+// ---- entry point that allocates nothing ---------------------------------------------------------------------
+// The split-K partial sums live in a file-scope device array instead of a caller's workspace.  In host code the
+// array's name is only a handle: its device address is looked up once per device and kept; every kernel argument
+// uses that address.
+namespace {
+
+static __device__ __align__(256) unsigned char scratch[SPMM_NOALLOC_SCRATCH_BYTES];
+
+constexpr int      kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+std::mutex         g_scratch_lock;
+
+// Device address of `scratch` on the current device, or nullptr (with *err set) when it cannot be found.
+void* scratch_address(hipError_t* err)
+{
+    int dev = -1;
+    *err    = hipGetDevice(&dev);
+    if (*err != hipSuccess)
+        return nullptr;
+    if (dev < 0 || dev >= kMaxDevices) {
+        *err = hipErrorInvalidDevice;
+        return nullptr;
+    }
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p != nullptr)
+        return p;
+    std::lock_guard<std::mutex> g(g_scratch_lock);
+    p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p != nullptr)
+        return p;
+    void* found = nullptr;
+    *err        = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (*err != hipSuccess || found == nullptr) {
+        if (*err == hipSuccess)
+            *err = hipErrorNotFound;
+        return nullptr;
+    }
+    g_scratch_ptr[dev].store(found, std::memory_order_release);
+    return found;
+}
+
+} // namespace
+
+extern "C" int SpMM_SplitK_API_NoAlloc(hipStream_t stream, const void* values, const uint64_t* bitmaps,
+                                       const int* offsets, const void* X, void* C, int M, int N, int K, int Split_K)
+{
+    if (int e = check_shape(M, N, K))
+        return e;
+    const int    sk   = Split_K <= 0 ? split_k_for(M, N, K) : clamp_split_k(Split_K, K);
+    const size_t need = sk > 1 ? sizeof(float) * (size_t)M * (size_t)N * (size_t)sk : 0;
+    if (need > (size_t)SPMM_NOALLOC_SCRATCH_BYTES) {
+        std::printf("MM_Sparse_API Error: M=%d N=%d Split_K=%d needs %zu bytes of partial sums; "
+                    "SpMM_SplitK_API_NoAlloc holds at most %zu!\n",
+                    M, N, sk, need, (size_t)SPMM_NOALLOC_SCRATCH_BYTES);
+        std::fflush(stdout);
+        return (int)hipErrorInvalidValue;
+    }
+    void* ws = nullptr;
+    if (sk > 1) {
+        hipError_t err = hipSuccess;
+        ws             = scratch_address(&err);
+        if (ws == nullptr) {
+            std::printf("MM_Sparse_API Error: the library's scratch array was not found on this device (%s)!\n",
+                        hipGetErrorString(err));
+            std::fflush(stdout);
+            return (int)err;
+        }
+    }
+    return run(stream, values, bitmaps, offsets, X, C, M, N, K, ws, sk, /*fp32_partials=*/true);
 }
 
 extern "C" void SpMM_TimeNextCall(hipEvent_t before_main, hipEvent_t after_main)

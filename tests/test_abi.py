@@ -10,6 +10,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def _declared_functions():
     text = open(os.path.join(ROOT, "include", "spmm_api.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"^[ \t]*#.*$", "", text, flags=re.M)  # preprocessor lines declare nothing
     c_part = text.split('} /* extern "C" */')[0] if '} /* extern "C" */' in text else text
     c_part = c_part.split("#ifdef __cplusplus\n}")[0]
     return sorted(set(re.findall(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\([^;{]*\)\s*;", c_part)))
@@ -21,7 +22,7 @@ def test_header_declares_the_expected_entry_points():
               "Our_GenSparseMatrixBinFile", "SpMM_SplitK_Auto", "SpMM_WorkspaceBytes", "SpMM_Version", "SpMM_TimeNextCall",
               "SpMM_SplitK_API_BiasAct", "SpMM_WorkspaceBytesBiasAct", "SpMM_EncodeDevice_Bitmaps",
               "SpMM_EncodeDevice_Values", "SpMM_SplitK_TableSet", "SpMM_SplitK_TableLoad", "SpMM_SplitK_TableSave",
-              "SpMM_SplitK_TableClear"):
+              "SpMM_SplitK_TableClear", "SpMM_SplitK_API_NoAlloc"):
         assert n in names
 
 
@@ -55,6 +56,10 @@ def test_shape_errors_are_reported_without_a_gpu(capfd):
     assert S.SpMM_SplitK_API(0, 0, 0, 0, 0, 0, 128, 16, 128, 0, 2) == 1  # split-K without a workspace
     assert S.SpMM_SplitK_API_BiasAct(0, 0, 0, 0, 0, 0, 64, 24, 64, 0, 1, 0, 0) == 999
     assert S.SpMM_SplitK_API_BiasAct(0, 0, 0, 0, 0, 0, 64, 16, 64, 0, 1, 0, 3) == 1  # unknown activation
+    capfd.readouterr()
+    assert S.SpMM_SplitK_API_NoAlloc(0, 0, 0, 0, 0, 0, 64, 24, 64, 1) == 999
+    assert S.SpMM_SplitK_API_NoAlloc(0, 0, 0, 0, 0, 0, 16384, 128, 4096, 8) == 1  # partial sums beyond the array
+    assert "holds at most" in capfd.readouterr().out
 
 
 def test_split_table_overrides_the_cost_model_and_round_trips_through_a_file(tmp_path):
