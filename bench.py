@@ -258,6 +258,22 @@ def decode_chain(torch, S, dev, layers, seed):
            "what": "ms per decode step over the linears of all layers; weights of every layer resident separately"}
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
+        # Before anything is timed: one pass of the chain, then every linear of the last layer recomputed in fp32
+        # from the dense weights on the very inputs the chain gave it (the buffers still hold that layer's values).
+        run_sparse(side)
+        side.synchronize()
+        j = layers - 1
+        x_in = hs[(j - 1) & 1] if j > 0 else h
+        worst = {"max_abs_frac": 0.0, "rel_l2": 0.0}
+        for nm, w, x, y in zip(names, dense[j], (x_in, attn, o, f), (qkv, o, f, hs[j & 1])):
+            ref = torch.matmul(x.float(), w.float().t())
+            d = (y.float() - ref)
+            worst["max_abs_frac"] = max(worst["max_abs_frac"], float(d.abs().max() / ref.abs().max()))
+            worst["rel_l2"] = max(worst["rel_l2"], float(d.norm() / ref.norm()))
+        out["check"] = dict(worst, what="last layer of the chain, every linear vs an fp32 product of the dense "
+                                        "weights with the chain's own inputs")
+        if not (worst["max_abs_frac"] <= 1e-2 and worst["rel_l2"] <= 1e-3):
+            raise RuntimeError(f"decode chain: outputs outside the tolerance: {worst}")
         out["sparse_eager_ms"] = timed(lambda: run_sparse(side), 5)
         out["dense_eager_ms"] = timed(lambda: run_dense(side), 5)
         for name, fn in (("sparse", run_sparse), ("dense", run_dense)):

@@ -106,13 +106,20 @@ def test_other_kernel_variants_match_oracle(torch, oracle, monkeypatch, variant)
         assert_spmm_close(C, _oracle_C(oracle, comp, X, sk, False), f"{variant} {M}x{K}x{N}")
 
 
+def _small_integer_problem(rng, M, K, N, density):
+    """Inputs whose products and partial sums are small integers: fp32 accumulation is exact in any order, so the
+    fp16 output is fixed bit for bit."""
+    W = rng.choice(np.array([-3, -2, -1, 1, 2, 3], np.float16), (M, K))
+    W[rng.random((M, K)) >= density] = 0
+    X = rng.integers(-2, 3, (N, K)).astype(np.float16)
+    return W, X
+
+
 def test_exact_on_small_integers(torch, oracle):
     """Where fp32 accumulation is exact the result must be bit-identical to the oracle, any Split_K."""
     rng = np.random.default_rng(5)
     M, K, N = 256, 512, 16
-    W = rng.integers(-3, 4, (M, K)).astype(np.float16)
-    W[rng.random((M, K)) < 0.6] = 0
-    X = rng.integers(-2, 3, (N, K)).astype(np.float16)
+    W, X = _small_integer_problem(rng, M, K, N, 0.4)
     comp = S.InitSparseMatrixA_bitmap(W)
     dev = Device(torch, comp)
     want = _oracle_C(oracle, comp, X).view(np.uint16)
@@ -120,6 +127,27 @@ def test_exact_on_small_integers(torch, oracle):
         for entry in ("api", "v3"):
             got = dev.spmm(X, sk, entry).view(np.uint16)
             assert np.array_equal(got, want), (sk, entry)
+
+
+@pytest.mark.parametrize("N", [8, 16, 32, 64, 128, 256])
+@pytest.mark.parametrize("density", [0.3, 0.85, 1.0])
+def test_exact_on_small_integers_every_width_and_dense_tiles(torch, oracle, N, density):
+    """Bit-identical results for every column-block width (N = 8 is the masked-column case of the 16-wide
+    kernel), for group tiles above 3072 values (density 0.85 and 1.0: their last value chunks are fetched when the
+    tile is staged), for the library's own Split_K and for explicit ones, through both entry points."""
+    rng = np.random.default_rng(100 + N)
+    M, K = 192, 640
+    W, X = _small_integer_problem(rng, M, K, N, density)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    if density >= 0.85:
+        assert comp.max_nnz > 3072
+    dev = Device(torch, comp)
+    want = _oracle_C(oracle, comp, X).view(np.uint16)
+    print(f"case N={N} density={density}", flush=True)
+    for sk in (0, 1, 3, 10):
+        assert np.array_equal(dev.spmm(X, sk, "api").view(np.uint16), want), ("api", sk)
+    for sk in (1, 5):
+        assert np.array_equal(dev.spmm(X, sk, "v3").view(np.uint16), want), ("v3", sk)
 
 
 def test_golden_fixtures_decode_on_device(torch, golden):
@@ -289,6 +317,117 @@ def test_opt30b_ffn1_full_size_other_batches_and_sparsities(torch, sparsity):
         ref = X.astype(np.float64) @ Wrows.T
         assert_spmm_close(dev.spmm(X, 0)[:, rows], ref, f"s={sparsity} N={N} auto")
         assert_spmm_close(dev.spmm(X, 2, "v3")[:, rows], ref, f"s={sparsity} N={N} v3 sk=2")
+
+
+@pytest.mark.parametrize("sparsity", [0.4, 0.5, 0.6, 0.7])
+def test_opt30b_ffn1_sweep_random_unstructured(torch, oracle, sparsity):
+    """The whole OPT-30B FFN1 sweep of the benchmark set: 28672x7168 with a uniform random mask at 40, 50, 60 and
+    70 % sparsity, N = 8, 16 and 32.  N = 16: the full output against the oracle; N = 8 and 32: sampled rows
+    against float64, automatic Split_K and an explicit one through the 14-argument entry point."""
+    M, K = 28672, 7168
+    W = make_weight(M, K, sparsity, seed=30 + int(sparsity * 10), pruning="random")
+    comp = S.InitSparseMatrixA_bitmap(W)
+    dev = Device(torch, comp)
+    rng = np.random.default_rng(17)
+    rows = rng.choice(M, 96, replace=False)
+    Wrows = W[rows].astype(np.float64)
+    del W
+    X = make_activations(K, 16, seed=16)
+    print(f"case s={sparsity} N=16 full output", flush=True)
+    want = _oracle_C(oracle, comp, X)
+    assert_spmm_close(dev.spmm(X, 0), want, f"s={sparsity} N=16 auto")
+    assert_spmm_close(want[:, rows], X.astype(np.float64) @ Wrows.T, "oracle vs float64")
+    for N in (8, 32):
+        X = make_activations(K, N, seed=N)
+        ref = X.astype(np.float64) @ Wrows.T
+        print(f"case s={sparsity} N={N}", flush=True)
+        assert_spmm_close(dev.spmm(X, 0)[:, rows], ref, f"s={sparsity} N={N} auto")
+        assert_spmm_close(dev.spmm(X, 3, "v3")[:, rows], ref, f"s={sparsity} N={N} v3 sk=3")
+
+
+OPT13B_LINEARS = [("opt13b_qkv", 15360, 5120), ("opt13b_out", 5120, 5120), ("opt13b_ffn1", 20480, 5120),
+                  ("opt13b_ffn2", 5120, 20480)]
+
+
+def _tuned_split(M, N, K):
+    """Split_K of the shipped measured table (spmspm_amd/tuned/), or None if the shape is not listed."""
+    path = os.path.join(os.path.dirname(S.__file__), "tuned", "splitk_mi355x_n16_s60.txt")
+    for line in open(path):
+        f = line.split()
+        if len(f) == 4 and not line.startswith("#") and (int(f[0]), int(f[1]), int(f[2])) == (M, N, K):
+            return int(f[3])
+    return None
+
+
+@pytest.mark.parametrize("name,M,K", OPT13B_LINEARS)
+def test_opt13b_decode_linears_full_size(torch, oracle, name, M, K):
+    """The four linears of an OPT-13B decode step at full size (60 % magnitude pruning, N = 16): the whole output
+    against the oracle with the library's own Split_K and with the shipped table's measured one."""
+    N = 16
+    W = make_weight(M, K, 0.6, seed=M // 64 + K // 64, pruning="magnitude")
+    X = make_activations(K, N, seed=5)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    del W
+    dev = Device(torch, comp)
+    want = _oracle_C(oracle, comp, X)
+    tuned = _tuned_split(M, N, K)
+    assert tuned is not None, "the shipped table lists every OPT-13B linear"
+    for sk in (0, tuned):
+        print(f"case {name} sk={sk}", flush=True)
+        assert_spmm_close(dev.spmm(X, sk), want, f"{name} sk={sk}")
+
+
+def test_opt13b_two_layer_chain_against_oracle(torch, oracle):
+    """Two OPT-13B-shaped layers chained on one stream the way the benchmark chains them (QKV, output projection on
+    a fixed attention result, FFN1, FFN2 feeding the next layer's QKV): every buffer of the chain against the
+    oracle run on the same inputs layer by layer."""
+    N = 16
+    rng = np.random.default_rng(77)
+    comps, lins = [], []
+    for layer in range(2):
+        row = []
+        for i, (name, M, K) in enumerate(OPT13B_LINEARS):
+            W = make_weight(M, K, 0.6, seed=500 + 10 * layer + i, pruning="magnitude")
+            # keep activations of order one down the chain: N(0, 0.02) weights shrink them by ~sqrt(0.4 K) * 0.02
+            W = (W.astype(np.float32) * np.float32(1.0 / (0.02 * np.sqrt(0.4 * K)))).astype(np.float16)
+            row.append(S.InitSparseMatrixA_bitmap(W))
+            del W
+        comps.append(row)
+        lins.append([S.SparseLinear(c, split_k=0) for c in row])
+    H = rng.uniform(-1, 1, (N, 5120)).astype(np.float16)
+    A = rng.uniform(-1, 1, (N, 5120)).astype(np.float16)
+    up = lambda a: torch.from_numpy(a.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+    h, attn = up(H), up(A)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    got = []
+    with torch.cuda.stream(side):
+        x = h
+        for lq, lo, l1, l2 in lins:
+            q = lq(x, stream=side)
+            o = lo(attn, stream=side)
+            f = l1(o, stream=side)
+            x = l2(f, stream=side)
+            got.append((q, o, f, x))
+    side.synchronize()
+
+    def ref(c, Xh):
+        Nn, Kk = Xh.shape
+        return oracle.spmm(c.values, c.bitmaps, c.offsets, Xh, c.M, Nn, Kk, S.SpMM_SplitK_Auto(c.M, Nn, Kk), False)
+
+    x_ref = H
+    for layer, ((cq, co, c1, c2), (q, o, f, x)) in enumerate(zip(comps, got)):
+        print(f"chain layer {layer}", flush=True)
+        # every linear is checked on the input the device actually gave it, so one rounding difference upstream
+        # does not decide the comparisons downstream; the chained buffers are compared as well
+        x_in = H if layer == 0 else got[layer - 1][3].cpu().numpy()
+        assert_spmm_close(q.cpu().numpy(), ref(cq, x_in), f"layer {layer} qkv")
+        assert_spmm_close(o.cpu().numpy(), ref(co, A), f"layer {layer} out-proj")
+        assert_spmm_close(f.cpu().numpy(), ref(c1, o.cpu().numpy()), f"layer {layer} ffn1")
+        assert_spmm_close(x.cpu().numpy(), ref(c2, f.cpu().numpy()), f"layer {layer} ffn2")
+        o_ref = ref(co, A)
+        x_ref = ref(c2, ref(c1, o_ref))
+        assert_spmm_close(x.cpu().numpy(), x_ref, f"layer {layer} chained output")
 
 
 def test_opt66b_ffn2_full_size_wide_batches(torch):
