@@ -336,11 +336,13 @@ class SparseLinear:
         self.nnz_padded = int(compressed.offsets[-1])
         self.split_k = split_k
         self._ws = None
+        self._plans = {}
 
     def clone(self):
         """A second resident copy of the same weights (device-to-device), e.g. one per decoder layer."""
         c = object.__new__(SparseLinear)
         c.M, c.K, c.device, c.nnz_padded, c.split_k, c._ws = self.M, self.K, self.device, self.nnz_padded, self.split_k, None
+        c._plans = {}
         c.activation, c.bias = self.activation, (None if self.bias is None else self.bias.clone())
         c.values, c.bitmaps, c.offsets = self.values.clone(), self.bitmaps.clone(), self.offsets.clone()
         return c
@@ -349,10 +351,25 @@ class SparseLinear:
         return (2 * self.nnz_padded + 8 * self.bitmaps.numel() + 4 * self.offsets.numel()
                 + 2 * self.K * N + 2 * self.M * N)
 
+    def _plan(self, N):
+        """(Split_K to pass, workspace bytes) for N columns.  An automatic Split_K is resolved here, once, and passed
+        on as an explicit value: the workspace is then sized for exactly the split the call will use, whatever
+        happens to the library's table afterwards, and the library is asked once per N instead of on every call."""
+        plan = self._plans.get(N)
+        if plan is None or plan[2] != self.split_k:
+            fused = self.bias is not None or self.activation != ACT_NONE
+            sk = self.split_k if self.split_k > 0 else SpMM_SplitK_Auto(self.M, N, self.K)
+            need = (SpMM_WorkspaceBytesBiasAct if fused else SpMM_WorkspaceBytes)(self.M, N, self.K, sk)
+            plan = self._plans[N] = (sk, need, self.split_k)
+        return plan
+
+    def replan(self):
+        """Forget resolved splits (after the library's Split_K table has changed)."""
+        self._plans = {}
+
     def workspace(self, N):
         import torch
-        fused = self.bias is not None or self.activation != ACT_NONE
-        need = (SpMM_WorkspaceBytesBiasAct if fused else SpMM_WorkspaceBytes)(self.M, N, self.K, self.split_k)
+        need = self._plan(N)[1]
         if need == 0:
             return None
         if self._ws is None or self._ws.numel() < need:
@@ -366,12 +383,13 @@ class SparseLinear:
             raise ValueError("x must be a contiguous [N][K] fp16 tensor")
         if out is None:
             out = torch.empty((N, self.M), dtype=torch.float16, device=self.device)
+        sk = self._plan(N)[0]
         if self.bias is not None or self.activation != ACT_NONE:
             err = SpMM_SplitK_API_BiasAct(stream, self.values, self.bitmaps, self.offsets, x, out, self.M, N, self.K,
-                                          self.workspace(N), self.split_k, self.bias, self.activation)
+                                          self.workspace(N), sk, self.bias, self.activation)
         else:
             err = SpMM_SplitK_API(stream, self.values, self.bitmaps, self.offsets, x, out, self.M, N, self.K,
-                                  self.workspace(N), self.split_k)
+                                  self.workspace(N), sk)
         if err != HIP_SUCCESS:
             raise RuntimeError(f"SpMM call failed with hipError_t {err}")
         return out

@@ -26,22 +26,32 @@ def hipcc():
     return exe
 
 
-def build_library(verbose=False, extra_flags=()):
+VARIANTS_LIBPATH = os.path.join(LIBDIR, "libSpMM_API_variants.so")
+
+
+def build_library(verbose=False, extra_flags=(), out=None):
     """Compile every source into one shared library.  Always recompiles."""
+    out = out or LIBPATH
     os.makedirs(LIBDIR, exist_ok=True)
     cmd = [hipcc(), *HIPCC_FLAGS, *extra_flags, "-I", os.path.join(ROOT, "include"), "-I", CSRC]
     cmd += [os.path.join(CSRC, s) for s in SOURCES]
-    cmd += ["-o", LIBPATH + ".tmp", "-lpthread"]
+    cmd += ["-o", out + ".tmp", "-lpthread"]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         sys.stderr.write(proc.stdout + proc.stderr)
-        raise RuntimeError("hipcc failed building libSpMM_API.so")
+        raise RuntimeError("hipcc failed building " + os.path.basename(out))
     if verbose and proc.stderr.strip():
         sys.stderr.write(proc.stderr)
-    os.replace(LIBPATH + ".tmp", LIBPATH)
-    return LIBPATH
+    os.replace(out + ".tmp", out)
+    return out
+
+
+def build_variants_library(verbose=False):
+    """The test build: the same library plus the two comparison kernels (-DSPMM_KEEP_VARIANTS) and the switch
+    SpMM_Debug_SetKernelVariant that selects them.  Only tests load it."""
+    return build_library(verbose=verbose, extra_flags=("-DSPMM_KEEP_VARIANTS",), out=VARIANTS_LIBPATH)
 
 
 HARNESS_SRC = os.path.join(ROOT, "tests", "cpp", "harness.cpp")
@@ -66,4 +76,5 @@ def build_harness(verbose=False):
 
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_variants_library(verbose=True))
     print(build_harness(verbose=True))

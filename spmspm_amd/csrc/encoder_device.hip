@@ -205,7 +205,11 @@ __global__ __launch_bounds__(kThreads) void encode_values(const uint16_t* __rest
     const int padded = (total + 7) & ~7;
     if (lane < padded - total)
         out[total + lane] = 0;
-    __builtin_amdgcn_wave_barrier(); // the wave's own LDS writes are ordered before its reads below
+    // the wave's own LDS writes are ordered before its reads below (lock step: no instruction; the fences hold the
+    // compiler to that order although the accesses alias through casts)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const int base = offsets[g];
     for (int i = lane; i < (padded >> 3); i += 64)
         reinterpret_cast<uint4*>(values + base)[i] = reinterpret_cast<const uint4*>(out)[i];

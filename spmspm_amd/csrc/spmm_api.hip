@@ -7,8 +7,10 @@
 #include <cstdio>
 #include <cstdlib>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <tuple>
+#include <vector>
 
 #include "spmm_api.h"
 #include "spmm_kernels.hiph"
@@ -69,10 +71,15 @@ int auto_split_k(int M, int N, int K)
 // end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:23, and of the SPLIT_K array of
 // kernel_benchmark/run_all_main.sh:5): a table keyed by (M, N, K), filled by SpMM_SplitK_TableSet or from a text
 // file of "M N K Split_K" lines.  SPMM_SPLITK_TABLE in the environment names a file that is loaded on first use.
+// Readers never lock: the table is an immutable snapshot behind an atomic pointer; a writer (rare: table set-up)
+// copies it under the mutex, changes the copy and publishes it.  Superseded snapshots stay alive until the process
+// ends, so a reader that still holds one is safe.
+using SplitMap = std::map<std::tuple<int, int, int>, int>;
 struct SplitTable {
-    std::mutex                                  lock;
-    std::map<std::tuple<int, int, int>, int>    entries;
-    bool                                        env_checked = false;
+    std::mutex                               lock;     // writers only
+    std::atomic<const SplitMap*>             current{nullptr};
+    std::vector<std::unique_ptr<SplitMap>>   versions; // every snapshot ever published (guarded by lock)
+    std::atomic<bool>                        env_checked{false};
 };
 SplitTable& split_table()
 {
@@ -80,14 +87,26 @@ SplitTable& split_table()
     return t;
 }
 
-// returns the number of entries read, or -1 when the file cannot be opened, -2 on a malformed line
+// Calls `change` on a private copy of the table and publishes the copy.  Caller holds t.lock.
+template <typename F>
+void publish_locked(SplitTable& t, F change)
+{
+    const SplitMap* cur = t.current.load(std::memory_order_acquire);
+    auto            nxt = std::make_unique<SplitMap>(cur ? *cur : SplitMap());
+    change(*nxt);
+    t.current.store(nxt.get(), std::memory_order_release);
+    t.versions.push_back(std::move(nxt));
+}
+
+// returns the number of entries read, or -1 when the file cannot be opened, -2 on a malformed line (nothing is
+// added then)
 int load_split_table_locked(SplitTable& t, const char* path)
 {
     std::FILE* f = std::fopen(path, "r");
     if (!f)
         return -1;
-    char line[256];
-    int  n = 0;
+    char     line[256];
+    SplitMap read;
     while (std::fgets(line, sizeof line, f)) {
         const char* p = line;
         while (*p == ' ' || *p == '\t')
@@ -99,34 +118,50 @@ int load_split_table_locked(SplitTable& t, const char* path)
             std::fclose(f);
             return -2;
         }
-        t.entries[std::make_tuple(m, nn, k)] = sk;
-        ++n;
+        read[std::make_tuple(m, nn, k)] = sk;
     }
     std::fclose(f);
-    return n;
+    publish_locked(t, [&](SplitMap& m) {
+        for (const auto& e : read)
+            m[e.first] = e.second;
+    });
+    return (int)read.size();
+}
+
+void check_env_table_once(SplitTable& t)
+{
+    if (t.env_checked.load(std::memory_order_acquire))
+        return;
+    std::lock_guard<std::mutex> g(t.lock);
+    if (t.env_checked.load(std::memory_order_relaxed))
+        return;
+    if (const char* e = std::getenv("SPMM_SPLITK_TABLE")) {
+        const int n = load_split_table_locked(t, e);
+        if (n < 0) {
+            std::printf("MM_Sparse_API Warning: SPMM_SPLITK_TABLE=%s %s; using the built-in choice.\n", e,
+                        n == -1 ? "cannot be opened" : "has a malformed line");
+            std::fflush(stdout);
+        }
+    }
+    t.env_checked.store(true, std::memory_order_release);
 }
 
 int split_k_for(int M, int N, int K)
 {
     SplitTable& t = split_table();
-    {
-        std::lock_guard<std::mutex> g(t.lock);
-        if (!t.env_checked) {
-            t.env_checked = true;
-            if (const char* e = std::getenv("SPMM_SPLITK_TABLE")) {
-                const int n = load_split_table_locked(t, e);
-                if (n < 0) {
-                    std::printf("MM_Sparse_API Warning: SPMM_SPLITK_TABLE=%s %s; using the built-in choice.\n", e,
-                                n == -1 ? "cannot be opened" : "has a malformed line");
-                    std::fflush(stdout);
-                }
-            }
-        }
-        auto it = t.entries.find(std::make_tuple(M, N, K));
-        if (it != t.entries.end())
+    check_env_table_once(t);
+    if (const SplitMap* m = t.current.load(std::memory_order_acquire)) {
+        auto it = m->find(std::make_tuple(M, N, K));
+        if (it != m->end())
             return clamp_split_k(it->second, K);
     }
-    return clamp_split_k(auto_split_k(M, N, K), K);
+    // the cost model's answer for the shape this thread asked about last is kept: a layer asks on every call
+    thread_local int last_m = 0, last_n = 0, last_k = 0, last_sk = 0;
+    if (M != last_m || N != last_n || K != last_k) {
+        last_sk = clamp_split_k(auto_split_k(M, N, K), K);
+        last_m = M, last_n = N, last_k = K;
+    }
+    return last_sk;
 }
 
 int check_shape(int M, int N, int K)
@@ -148,10 +183,20 @@ int check_shape(int M, int N, int K)
 thread_local hipEvent_t t_before_main = nullptr;
 thread_local hipEvent_t t_after_main  = nullptr;
 
+// An entry point that refuses its arguments before run() is reached drops the timing request too.
+int refuse(int error)
+{
+    t_before_main = t_after_main = nullptr;
+    return error;
+}
+
 int run(hipStream_t stream, const void* values, const uint64_t* bitmaps, const int* offsets, const void* X, void* C,
         int M, int N, int K, void* workspace, int split_k, bool fp32_partials, bool epilogue = false,
         const void* bias = nullptr, int act = 0)
 {
+    // the timing request belongs to this call whatever becomes of it
+    hipEvent_t before = t_before_main, after = t_after_main;
+    t_before_main = t_after_main = nullptr;
     if (int e = check_shape(M, N, K))
         return e;
     split_k = clamp_split_k(split_k, K);
@@ -160,16 +205,13 @@ int run(hipStream_t stream, const void* values, const uint64_t* bitmaps, const i
         std::fflush(stdout);
         return (int)hipErrorInvalidValue;
     }
-    (void)hipGetLastError(); // do not report a stale error as ours
-    hipEvent_t before = t_before_main, after = t_after_main;
-    t_before_main = t_after_main = nullptr;
-    spmm::launch_spmm(stream, static_cast<const __half*>(values), bitmaps, offsets, static_cast<const __half*>(X),
-                      static_cast<__half*>(C), M, N, K, workspace, split_k, fp32_partials, before, after, epilogue);
-    hipError_t err = hipGetLastError();
+    hipError_t err = spmm::launch_spmm(stream, static_cast<const __half*>(values), bitmaps, offsets,
+                                       static_cast<const __half*>(X), static_cast<__half*>(C), M, N, K, workspace,
+                                       split_k, fp32_partials, before, after, epilogue);
     if (err != hipSuccess || (split_k == 1 && !epilogue))
         return (int)err;
-    spmm::launch_reduction(stream, static_cast<__half*>(C), workspace, M, N, split_k, fp32_partials, bias, act);
-    return (int)hipGetLastError();
+    return (int)spmm::launch_reduction(stream, static_cast<__half*>(C), workspace, M, N, split_k, fp32_partials, bias,
+                                       act);
 }
 
 } // namespace
@@ -187,7 +229,7 @@ extern "C" int SpMM_SplitK_TableSet(int M, int N, int K, int Split_K)
         return (int)hipErrorInvalidValue;
     SplitTable&                 t = split_table();
     std::lock_guard<std::mutex> g(t.lock);
-    t.entries[std::make_tuple(M, N, K)] = Split_K;
+    publish_locked(t, [&](SplitMap& m) { m[std::make_tuple(M, N, K)] = Split_K; });
     return 0;
 }
 
@@ -204,23 +246,26 @@ extern "C" int SpMM_SplitK_TableSave(const char* path)
 {
     if (path == nullptr)
         return -1;
-    SplitTable&                 t = split_table();
-    std::lock_guard<std::mutex> g(t.lock);
-    std::FILE*                  f = std::fopen(path, "w");
+    const SplitMap* m = split_table().current.load(std::memory_order_acquire);
+    std::FILE*      f = std::fopen(path, "w");
     if (!f)
         return -1;
     std::fprintf(f, "# M N K Split_K\n");
-    for (const auto& e : t.entries)
-        std::fprintf(f, "%d %d %d %d\n", std::get<0>(e.first), std::get<1>(e.first), std::get<2>(e.first), e.second);
+    int n = 0;
+    if (m)
+        for (const auto& e : *m) {
+            std::fprintf(f, "%d %d %d %d\n", std::get<0>(e.first), std::get<1>(e.first), std::get<2>(e.first), e.second);
+            ++n;
+        }
     std::fclose(f);
-    return (int)t.entries.size();
+    return n;
 }
 
 extern "C" void SpMM_SplitK_TableClear(void)
 {
     SplitTable&                 t = split_table();
     std::lock_guard<std::mutex> g(t.lock);
-    t.entries.clear();
+    publish_locked(t, [](SplitMap& m) { m.clear(); });
 }
 
 extern "C" size_t SpMM_WorkspaceBytes(int M, int N, int K, int Split_K)
@@ -236,9 +281,7 @@ extern "C" size_t SpMM_WorkspaceBytes(int M, int N, int K, int Split_K)
 extern "C" int SpMM_SplitK_API(hipStream_t stream, const void* values, const uint64_t* bitmaps, const int* offsets,
                                const void* X, void* C, int M, int N, int K, void* workspace, int Split_K)
 {
-    if (int e = check_shape(M, N, K))
-        return e;
-    int sk = Split_K <= 0 ? SpMM_SplitK_Auto(M, N, K) : Split_K;
+    const int sk = Split_K <= 0 ? SpMM_SplitK_Auto(M, N, K) : Split_K; // 1 for a shape that run() will refuse
     return run(stream, values, bitmaps, offsets, X, C, M, N, K, workspace, sk, /*fp32_partials=*/true);
 }
 
@@ -255,11 +298,11 @@ extern "C" int SpMM_SplitK_API_BiasAct(hipStream_t stream, const void* values, c
                                        void* workspace, int Split_K, const void* bias, int activation)
 {
     if (int e = check_shape(M, N, K))
-        return e;
+        return refuse(e);
     if (activation < 0 || activation > 2) {
         std::printf("MM_Sparse_API Error: unknown activation %d (0 none, 1 ReLU, 2 GELU)!\n", activation);
         std::fflush(stdout);
-        return (int)hipErrorInvalidValue;
+        return refuse((int)hipErrorInvalidValue);
     }
     int sk = Split_K <= 0 ? SpMM_SplitK_Auto(M, N, K) : Split_K;
     return run(stream, values, bitmaps, offsets, X, C, M, N, K, workspace, sk, /*fp32_partials=*/true,
@@ -273,11 +316,11 @@ extern "C" int SpMM_SplitK_API_bitmap_v3(hipStream_t stream, const void* /*A*/, 
                                          void* Reduction_Workspace, int Split_K)
 {
     if (int e = check_shape(M_Global, N_Global, K_Global))
-        return e;
+        return refuse(e);
     if (Split_K < 1) {
         std::printf("MM_Sparse_API Error: Split_K (%d) must be >= 1!\n", Split_K);
         std::fflush(stdout);
-        return (int)hipErrorInvalidValue;
+        return refuse((int)hipErrorInvalidValue);
     }
     return run(stream, Compressed_A, bitmap, TileOffsets, B, C, M_Global, N_Global, K_Global, Reduction_Workspace,
                Split_K, /*fp32_partials=*/false);
@@ -330,7 +373,7 @@ extern "C" int SpMM_SplitK_API_NoAlloc(hipStream_t stream, const void* values, c
                                        const int* offsets, const void* X, void* C, int M, int N, int K, int Split_K)
 {
     if (int e = check_shape(M, N, K))
-        return e;
+        return refuse(e);
     const int    sk   = Split_K <= 0 ? split_k_for(M, N, K) : clamp_split_k(Split_K, K);
     const size_t need = sk > 1 ? sizeof(float) * (size_t)M * (size_t)N * (size_t)sk : 0;
     if (need > (size_t)SPMM_NOALLOC_SCRATCH_BYTES) {
@@ -338,7 +381,7 @@ extern "C" int SpMM_SplitK_API_NoAlloc(hipStream_t stream, const void* values, c
                     "SpMM_SplitK_API_NoAlloc holds at most %zu!\n",
                     M, N, sk, need, (size_t)SPMM_NOALLOC_SCRATCH_BYTES);
         std::fflush(stdout);
-        return (int)hipErrorInvalidValue;
+        return refuse((int)hipErrorInvalidValue);
     }
     void* ws = nullptr;
     if (sk > 1) {
@@ -348,7 +391,7 @@ extern "C" int SpMM_SplitK_API_NoAlloc(hipStream_t stream, const void* values, c
             std::printf("MM_Sparse_API Error: the library's scratch array was not found on this device (%s)!\n",
                         hipGetErrorString(err));
             std::fflush(stdout);
-            return (int)err;
+            return refuse((int)err);
         }
     }
     return run(stream, values, bitmaps, offsets, X, C, M, N, K, ws, sk, /*fp32_partials=*/true);
@@ -359,6 +402,14 @@ extern "C" void SpMM_TimeNextCall(hipEvent_t before_main, hipEvent_t after_main)
     t_before_main = before_main;
     t_after_main  = after_main;
 }
+
+#ifdef SPMM_KEEP_VARIANTS
+// Test build only (not in the header): selects the comparison kernel for the calls that follow.
+extern "C" void SpMM_Debug_SetKernelVariant(int variant)
+{
+    spmm::kernel_variant() = variant;
+}
+#endif
 
 extern "C" const char* SpMM_Version(void)
 {

@@ -72,6 +72,24 @@ def tune_shape(M, N, K, sparsity=0.6, candidates=None, device="cuda:0", iters=30
     return best, times
 
 
+def _cost_model_choice(M, N, K):
+    """What the built-in cost model picks for a shape, with the table left exactly as it was: the table is saved
+    to a temporary file, emptied for the question and loaded back (entries of the user, of SPMM_SPLITK_TABLE and of
+    earlier shapes alike)."""
+    import os
+    import tempfile
+    fd, path = tempfile.mkstemp(suffix=".splitk")
+    os.close(fd)
+    try:
+        A.SpMM_SplitK_TableSave(path)
+        A.SpMM_SplitK_TableClear()
+        model = A.SpMM_SplitK_Auto(M, N, K)
+        A.SpMM_SplitK_TableLoad(path)
+    finally:
+        os.unlink(path)
+    return model
+
+
 def tune(shapes, N, sparsity=0.6, record=True, log=None, **kw):
     """tune_shape over (M, K) pairs; with `record`, each winner goes into the library's table.
     Returns {(M, N, K): (best, times)}."""
@@ -82,12 +100,7 @@ def tune(shapes, N, sparsity=0.6, record=True, log=None, **kw):
         if record:
             A.SpMM_SplitK_TableSet(M, N, K, best)
         if log:
-            model = None
-            if record:
-                A.SpMM_SplitK_TableClear()
-                model = A.SpMM_SplitK_Auto(M, N, K)
-                for (m, n, k), (b, _) in out.items():
-                    A.SpMM_SplitK_TableSet(m, n, k, b)
+            model = _cost_model_choice(M, N, K) if record else None
             log(f"M={M} N={N} K={K}: best Split_K {best} ({times[best]:.1f} us)"
                 + (f", cost model {model} ({times.get(model, float('nan')):.1f} us)" if model else "")
                 + "  " + " ".join(f"{s}:{t:.1f}" for s, t in sorted(times.items())))

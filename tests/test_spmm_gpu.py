@@ -93,17 +93,40 @@ def test_matches_oracle(torch, oracle, M, K, N, s, sk):
     assert_spmm_close(Cv3, ref64, "v3 vs float64")
 
 
-@pytest.mark.parametrize("variant", ["baseline", "stream"])
-def test_other_kernel_variants_match_oracle(torch, oracle, monkeypatch, variant):
-    """The comparison kernels (simple staging kernel, lane-per-bit decode through a dense LDS tile) stay correct."""
-    monkeypatch.setenv("SPMM_KERNEL", variant)
-    for M, K, N, s, sk in [(128, 192, 16, 0.7, 1), (256, 1024, 8, 0.6, 3), (128, 512, 64, 0.5, 2), (256, 256, 32, 0.0, 1)]:
-        W = make_weight(M, K, s, seed=M + K + N)
-        X = make_activations(K, N, seed=N)
-        comp = S.InitSparseMatrixA_bitmap(W)
-        print(f"case {variant} M={M} K={K} N={N} sk={sk}", flush=True)
-        C = Device(torch, comp).spmm(X, sk, "api")
-        assert_spmm_close(C, _oracle_C(oracle, comp, X, sk, False), f"{variant} {M}x{K}x{N}")
+@pytest.mark.parametrize("variant", [0, 1, 2], ids=["baseline", "stream", "rows"])
+def test_other_kernel_variants_match_oracle(torch, oracle, variant):
+    """The comparison kernels (simple staging kernel, lane-per-bit decode through a dense LDS tile) stay correct.
+    They live in the test build of the library only (libSpMM_API_variants.so, -DSPMM_KEEP_VARIANTS), which also has
+    the switch that selects them; the shipped library has neither."""
+    import ctypes as C
+    path = os.path.join(os.path.dirname(S.library_path()), "libSpMM_API_variants.so")
+    assert os.path.exists(path), "build it with __graft_entry__.build()"
+    assert not hasattr(S.library(), "SpMM_Debug_SetKernelVariant")
+    L = C.CDLL(path)
+    L.SpMM_SplitK_API.restype = C.c_int
+    L.SpMM_SplitK_API.argtypes = [C.c_void_p] * 6 + [C.c_int] * 3 + [C.c_void_p, C.c_int]
+    L.SpMM_Debug_SetKernelVariant.argtypes = [C.c_int]
+    L.SpMM_Debug_SetKernelVariant(variant)
+    try:
+        for M, K, N, s, sk in [(128, 192, 16, 0.7, 1), (256, 1024, 8, 0.6, 3), (128, 512, 64, 0.5, 2),
+                               (256, 256, 32, 0.0, 1)]:
+            W = make_weight(M, K, s, seed=M + K + N)
+            X = make_activations(K, N, seed=N)
+            comp = S.InitSparseMatrixA_bitmap(W)
+            dev = Device(torch, comp)
+            print(f"case variant {variant} M={M} K={K} N={N} sk={sk}", flush=True)
+            x = torch.from_numpy(X.view(np.int16).copy()).to("cuda:0")
+            out = torch.full((N, M), 0x7e00, dtype=torch.int16, device="cuda:0")
+            ws = torch.empty(max(4 * M * N * sk, 16), dtype=torch.uint8, device="cuda:0")
+            err = L.SpMM_SplitK_API(torch.cuda.current_stream().cuda_stream, dev.values.data_ptr(),
+                                    dev.bitmaps.data_ptr(), dev.offsets.data_ptr(), x.data_ptr(), out.data_ptr(),
+                                    M, N, K, ws.data_ptr(), sk)
+            assert err == 0
+            torch.cuda.synchronize()
+            C_out = out.cpu().numpy().view(np.float16)
+            assert_spmm_close(C_out, _oracle_C(oracle, comp, X, sk, False), f"variant {variant} {M}x{K}x{N}")
+    finally:
+        L.SpMM_Debug_SetKernelVariant(2)
 
 
 def _small_integer_problem(rng, M, K, N, density):
