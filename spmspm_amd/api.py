@@ -347,6 +347,13 @@ class SparseLinear:
         c.values, c.bitmaps, c.offsets = self.values.clone(), self.bitmaps.clone(), self.offsets.clone()
         return c
 
+    def module(self):
+        """The same resident weights as a `torch.nn.Module` whose forward is the registered operator
+        `torch.ops.spmspm_amd.sparse_linear` (spmspm_amd/torch_ops.py): traceable by torch.compile, usable in
+        nn.Sequential, capturable in graphs.  Shares this layer's device arrays."""
+        from .torch_ops import SparseLinearModule
+        return SparseLinearModule.from_layer(self)
+
     def bytes_per_call(self, N):
         return (2 * self.nnz_padded + 8 * self.bitmaps.numel() + 4 * self.offsets.numel()
                 + 2 * self.K * N + 2 * self.M * N)
