@@ -7,8 +7,9 @@ A step is one SpMM call (main kernel + split-K reduction when the library's
 automatic Split_K is > 1) over one resident compressed copy of the weight
 matrix.  Calls rotate over enough copies of the weights that successive steps
 cannot be served from the 256 MB last-level cache.  Prints one JSON line:
-dense-equivalent TFLOP/s as `value`, plus `roofline` (HBM, algorithmic bytes
-over the main kernel's event-timed duration) and `cpu_baseline` (the CPU
+dense-equivalent TFLOP/s as `value`, plus `roofline` (HBM: algorithmic bytes
+over the GPU time of one whole call, with the main kernel alone and this
+machine's own read-stream ceiling beside it) and `cpu_baseline` (the CPU
 checker timed on this machine's host cores over a bounded row slice).
 """
 import argparse
@@ -47,6 +48,8 @@ def parse():
     p.add_argument("--no-chain", action="store_true",
                    help="skip the OPT-13B decode-step chain (40 layers x 4 linears, sparse vs dense, same run)")
     p.add_argument("--chain-layers", type=int, default=40)
+    p.add_argument("--no-stream-probe", action="store_true",
+                   help="skip the read-stream probe (spmspm_amd/lib/stream_probe) behind roofline.stream_ceiling_gbs")
     p.add_argument("--copy-probe", action="store_true",
                    help="also run three 256 MiB device-to-device copies (a known-size reference for HBM byte counters)")
     return p.parse_args()
@@ -172,7 +175,8 @@ def quick_measure(torch, S, hip, dev, workload, steps, warmup, seed):
     flops = 2.0 * M * N * K
     return {"workload": workload, "M": M, "K": K, "N": N, "sparsity": w["sparsity"], "pruning": w["pruning"],
             "split_k": S.SpMM_SplitK_Auto(M, N, K), "tflops": flops / wall / 1e12, "us_per_call": wall * 1e6,
-            "kernel_avg_us": kern * 1e6, "gbs": algo / kern / 1e9, "roofline_frac": algo / kern / 1e9 / HBM_PEAK_GBS,
+            "kernel_avg_us": kern * 1e6, "gbs": algo / wall / 1e9, "roofline_frac": algo / wall / 1e9 / HBM_PEAK_GBS,
+            "main_kernel_gbs": algo / kern / 1e9, "main_kernel_roofline_frac": algo / kern / 1e9 / HBM_PEAK_GBS,
             "algorithmic_bytes": int(algo), "dense_fp16_us": td * 1e6, "speedup_vs_dense": td / wall,
             "rel_l2": float(np.linalg.norm(got - ref) / np.linalg.norm(ref))}
 
@@ -356,12 +360,17 @@ def main():
         step(i)
     torch.cuda.synchronize()
 
-    # timed region 1: K steps, wall clock between synchronisations -> value
+    # timed region 1: K steps, wall clock between synchronisations -> value; the same steps on the GPU's clock
+    # (events recorded on the launch stream before the first and after the last call) -> roofline
+    g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    g0.record(stream)
     for i in range(a.steps):
         step(i)
+    g1.record(stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    call_gpu_s = g0.elapsed_time(g1) / 1e3 / a.steps
 
     # timed region 2: the same K steps with a HIP event pair attached to every main-kernel dispatch -> roofline
     events = [(hip.event(), hip.event()) for _ in range(a.steps)]
@@ -384,7 +393,8 @@ def main():
     flops = 2.0 * M * N * K
     value = flops / (wall / a.steps) / 1e12
     kern_avg_s = float(kern_ms.mean()) / 1e3
-    achieved = algo_bytes / kern_avg_s / 1e9
+    achieved = algo_bytes / call_gpu_s / 1e9          # whole call: main kernel + split-K reduction + the gap between
+    achieved_main = algo_bytes / kern_avg_s / 1e9     # main kernel alone
 
     # correctness of what was timed: a row sample against float64
     rows = np.random.default_rng(1).choice(M, 128, replace=False)
@@ -409,12 +419,28 @@ def main():
                  "what": "torch.matmul fp16 (hipBLASLt), same run, rotating weight copies"}
         del Wd
 
-    traffic = None
+    # HBM bytes per launch of the main kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE.  The record
+    # is only quoted when it was taken for exactly what ran here: same workload, width, sparsity, Split_K, kernel.
+    nt = 1 if N <= 16 else (2 if N == 32 else 4)
+    kernel_name = f"spmm::spmm_bitmap_rows<{nt}, {'true' if split_k > 1 else 'false'}>"
+    traffic, traffic_note = None, "no record for this configuration in profiles/traffic.json"
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):  # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+    if os.path.exists(tpath):
         rec = json.load(open(tpath)).get(f"{a.workload}_n{N}_s{int(round(w['sparsity'] * 100))}")
-        if rec:
-            traffic = rec["bytes_per_launch"]
+        if rec and rec.get("split_k") == split_k and rec.get("kernel") == kernel_name:
+            traffic, traffic_note = rec["bytes_per_launch"], rec["source"]
+        elif rec:
+            traffic_note = (f"record is for {rec.get('kernel')} at Split_K={rec.get('split_k')}, this run used "
+                            f"{kernel_name} at Split_K={split_k}: not quoted")
+
+    stream_ceiling = None
+    probe = os.path.join(os.path.dirname(S.library_path()), "stream_probe")
+    if not a.no_stream_probe and os.path.exists(probe):
+        import subprocess
+        pr = subprocess.run([probe], capture_output=True, text=True, timeout=120)
+        for line in pr.stdout.splitlines():
+            if line.startswith("{"):
+                stream_ceiling = json.loads(line)
 
     out = {
         "metric": "SpMM dense-equiv TFLOP/s", "value": value, "unit": "TFLOP/s", "n_gpus": 1,
@@ -427,11 +453,22 @@ def main():
                    "workspace_bytes": ws_bytes},
         "gbs_whole_call": algo_bytes / (wall / a.steps) / 1e9,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "algorithmic_bytes_per_launch": algo_bytes, "kernel": "spmm main kernel",
-                     "kernel_avg_us": kern_avg_s * 1e6, "kernel_min_us": float(kern_ms.min()) * 1e3,
-                     "timing": "HIP events attached to each main-kernel dispatch (kernel begin/end timestamps), "
-                               "same K steps repeated after the wall-clock region"},
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": traffic_note,
+                     "algorithmic_bytes_per_launch": algo_bytes,
+                     "what": "algorithmic bytes / GPU time of one call (main kernel + split-K reduction and the gap "
+                             "between them), from events recorded on the launch stream around the K timed steps",
+                     "call_us": call_gpu_s * 1e6,
+                     "main_kernel": {"name": kernel_name, "avg_us": kern_avg_s * 1e6,
+                                     "min_us": float(kern_ms.min()) * 1e3, "achieved": achieved_main,
+                                     "frac": achieved_main / HBM_PEAK_GBS,
+                                     "timing": "HIP events attached to each main-kernel dispatch (kernel begin/end "
+                                               "timestamps), the same K steps repeated after the first region"},
+                     "stream_ceiling_gbs": None if stream_ceiling is None else stream_ceiling["stream_ceiling_gbs"],
+                     "frac_of_stream_ceiling": None if stream_ceiling is None
+                     else achieved / stream_ceiling["stream_ceiling_gbs"],
+                     "stream_ceiling_what": None if stream_ceiling is None
+                     else "best plain read stream of this GPU in this run (spmspm_amd/lib/stream_probe): "
+                          + stream_ceiling["best"]},
         "check": {"max_abs_over_max_ref": max_abs_frac, "rel_l2": rel_l2, "rows_sampled": 128},
         "dense_fp16": dense,
         "host": {"generate_s": t_gen, "encode_s": t_enc, "encode_threads": os.cpu_count()},

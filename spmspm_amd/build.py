@@ -74,7 +74,27 @@ def build_harness(verbose=False):
     return HARNESS_PATH
 
 
+PROBE_SRC = os.path.join(CSRC, "stream_probe.hip")
+PROBE_PATH = os.path.join(LIBDIR, "stream_probe")
+
+
+def build_stream_probe(verbose=False):
+    """The read-streaming probe (csrc/stream_probe.hip): a stand-alone program bench.py runs to put the machine's
+    own read ceiling next to the data-sheet peak."""
+    cmd = [hipcc(), "-O3", "-std=c++17", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-Wno-unused-command-line-argument", PROBE_SRC, "-o", PROBE_PATH + ".tmp"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        sys.stderr.write(proc.stdout + proc.stderr)
+        raise RuntimeError("hipcc failed building the stream probe")
+    os.replace(PROBE_PATH + ".tmp", PROBE_PATH)
+    return PROBE_PATH
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
     print(build_variants_library(verbose=True))
     print(build_harness(verbose=True))
+    print(build_stream_probe(verbose=True))
