@@ -31,6 +31,37 @@ int clamp_split_k(int split_k, int K)
     return split_k < 1 ? 1 : split_k;
 }
 
+// K split of the wide kernel (N a multiple of 128, spmm_kernel_wide.hiph).  A workgroup covers 256 rows x 128 columns
+// x one K batch and two workgroups fit a CU, so the 512 slots are the unit: one round of at most 512 workgroups,
+// each walking ceil(nkb / split) k blocks plus a start-up of about two.  Measured on OPT-66B FFN2 (9216 x 36864,
+// N = 128): a workgroup alone on its CU takes 2.2 us per k block, two sharing a CU 3.45 us each (ratio 1.57);
+// Split_K 7 / 12 / 14 / 16 -> 252 / 432 / 504 / 576 workgroups -> 177 / 151 / 141 / 177 us.  The partial slabs of a
+// split are re-read from cache by the reduction, which adds little.
+int auto_split_k_wide(int M, int N, int K)
+{
+    const int    nkb  = K / 64;
+    const long   base = (long)((M / 64 + 3) / 4) * (N / 128);
+    const double kSlots = 512.0, kAloneSlots = 256.0, kShared = 1.57, kStartup = 2.0;
+    int          best = 1;
+    double       best_c = 1e30;
+    int          max_sk = nkb / 2 > 0 ? nkb / 2 : 1; // at least two k blocks per batch
+    if (max_sk > 32)
+        max_sk = 32;
+    for (int sk = 1; sk <= max_sk; ++sk) {
+        const double wgs    = (double)base * sk;
+        const double rounds = (double)((long)((wgs + kSlots - 1) / kSlots));
+        const double steps  = (double)((nkb + sk - 1) / sk) + kStartup;
+        double       cost   = rounds * steps * (wgs > kAloneSlots ? kShared : 1.0);
+        if (sk > 1)
+            cost += 1.0 + sk * ((double)M * N * 8.0) / 8e12 / 2.2e-6;
+        if (cost < best_c - 1e-9) {
+            best_c = cost;
+            best   = sk;
+        }
+    }
+    return best;
+}
+
 // Picks the K split from a small cost model (units: group tiles processed by the busiest CU), fitted to whole-call
 // times (main kernel + reduction, back to back on one stream) of ten OPT-like shapes at Split_K 1..20, where its
 // choice is within 4 % of the best measured split:
@@ -39,6 +70,8 @@ int clamp_split_k(int split_k, int K)
 //   partials a split adds the reduction kernel, and every batch writes and re-reads an fp32 slab of M*N.
 int auto_split_k(int M, int N, int K)
 {
+    if (spmm::use_wide_kernel(M, N))
+        return auto_split_k_wide(M, N, K);
     const int    nkb  = K / 64;
     const long   base = (long)(M / 64) * spmm::column_blocks(N);
     const double kCUs = 256.0, kStartupTiles = 2.0, kFillWGsPerCU = 2.0, kReductionTiles = 2.0, kTileBytes = 2000.0;

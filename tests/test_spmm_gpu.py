@@ -93,9 +93,11 @@ def test_matches_oracle(torch, oracle, M, K, N, s, sk):
     assert_spmm_close(Cv3, ref64, "v3 vs float64")
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2], ids=["baseline", "stream", "rows"])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4], ids=["baseline", "stream", "shipped", "rows-everywhere", "wide-everywhere"])
 def test_other_kernel_variants_match_oracle(torch, oracle, variant):
-    """The comparison kernels (simple staging kernel, lane-per-bit decode through a dense LDS tile) stay correct.
+    """The comparison kernels (simple staging kernel, lane-per-bit decode through a dense LDS tile) stay correct, and
+    so do the row-per-lane kernel at N >= 128 and the wide kernel at N = 64 and on fewer than 256 rows, which the
+    shipped dispatch does not use there.
     They live in the test build of the library only (libSpMM_API_variants.so, -DSPMM_KEEP_VARIANTS), which also has
     the switch that selects them; the shipped library has neither."""
     import ctypes as C
@@ -109,7 +111,8 @@ def test_other_kernel_variants_match_oracle(torch, oracle, variant):
     L.SpMM_Debug_SetKernelVariant(variant)
     try:
         for M, K, N, s, sk in [(128, 192, 16, 0.7, 1), (256, 1024, 8, 0.6, 3), (128, 512, 64, 0.5, 2),
-                               (256, 256, 32, 0.0, 1)]:
+                               (256, 256, 32, 0.0, 1), (320, 704, 64, 0.5, 3), (128, 512, 128, 0.6, 2),
+                               (576, 384, 256, 0.3, 1)]:
             W = make_weight(M, K, s, seed=M + K + N)
             X = make_activations(K, N, seed=N)
             comp = S.InitSparseMatrixA_bitmap(W)
@@ -170,6 +173,37 @@ def test_exact_on_small_integers_every_width_and_dense_tiles(torch, oracle, N, d
     for sk in (0, 1, 3, 10):
         assert np.array_equal(dev.spmm(X, sk, "api").view(np.uint16), want), ("api", sk)
     for sk in (1, 5):
+        assert np.array_equal(dev.spmm(X, sk, "v3").view(np.uint16), want), ("v3", sk)
+
+
+WIDE_CASES = [
+    # M, K, N, density, explicit splits
+    (256, 512, 128, 0.5, (1, 2, 8)),      # one workgroup per batch; Split_K = 8 leaves one k block per batch
+    (320, 576, 128, 0.6, (1, 4)),         # five row blocks: the second workgroup has one wave with a row block;
+                                          # nine k blocks in four batches: the last batch is empty
+    (832, 1536, 256, 0.9, (1, 2, 5)),     # two column groups of 128; tiles above 3072 values
+    (512, 1024, 128, 1.0, (1, 3)),        # every tile full: the last value chunks are fetched when the tile is staged
+    (1024, 4096, 128, 0.05, (1, 2, 7)),   # nearly empty tiles, fewer value chunks than registers for them
+    (256, 128, 384, 0.4, (1, 2)),         # two k blocks, three column groups
+]
+
+
+@pytest.mark.parametrize("M,K,N,density,splits", WIDE_CASES)
+def test_wide_kernel_exact_on_small_integers(torch, oracle, M, K, N, density, splits):
+    """N a multiple of 128 and M >= 256 run on the wide kernel (a group tile decoded once per 128 columns, X staged
+    in LDS per workgroup).  Bit-identical to the oracle where fp32 accumulation is exact: the library's own Split_K
+    and explicit ones, fp32 partial slabs ("api") and fp16 ones ("v3")."""
+    rng = np.random.default_rng(M + K + N)
+    W, X = _small_integer_problem(rng, M, K, N, density)
+    W[64:128, :] = 0                      # an all-zero row block
+    W[:, 64:128] = 0                      # and an all-zero column of group tiles
+    comp = S.InitSparseMatrixA_bitmap(W)
+    dev = Device(torch, comp)
+    want = _oracle_C(oracle, comp, X).view(np.uint16)
+    for sk in (0,) + tuple(splits):
+        print(f"case wide M={M} K={K} N={N} density={density} sk={sk}", flush=True)
+        assert np.array_equal(dev.spmm(X, sk, "api").view(np.uint16), want), ("api", sk)
+    for sk in splits[:2]:
         assert np.array_equal(dev.spmm(X, sk, "v3").view(np.uint16), want), ("v3", sk)
 
 
@@ -548,7 +582,8 @@ def test_calls_recorded_in_a_hip_graph_replay_correctly(torch, oracle):
 
 
 @pytest.mark.parametrize("M,K,N,s,sk", [(256, 512, 16, 0.6, 1), (512, 1024, 8, 0.7, 4), (1024, 256, 32, 0.5, 0),
-                                        (320, 4096, 64, 0.6, 0), (128, 128, 128, 0.3, 2)])
+                                        (320, 4096, 64, 0.6, 0), (128, 128, 128, 0.3, 2), (512, 768, 128, 0.6, 1),
+                                        (320, 1024, 256, 0.5, 3)])
 @pytest.mark.parametrize("act", [0, 1, 2])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_bias_activation_entry_point(torch, oracle, M, K, N, s, sk, act, with_bias):
