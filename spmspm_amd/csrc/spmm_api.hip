@@ -209,6 +209,11 @@ int check_shape(int M, int N, int K)
         std::fflush(stdout);
         return (int)hipErrorInvalidValue;
     }
+    if (M / 64 > 65535) { // row blocks are the z dimension of the launch grid
+        std::printf("MM_Sparse_API Error: M (%d) exceeds 64 * 65535 rows!\n", M);
+        std::fflush(stdout);
+        return (int)hipErrorInvalidValue;
+    }
     return 0;
 }
 
