@@ -67,6 +67,18 @@ int SpMM_SplitK_API(hipStream_t stream, const void* values, const uint64_t* bitm
                     const void* X, void* C, int M, int N, int K, void* workspace, int Split_K);
 
 /*
+ * SpMM_SplitK_API with the size of `workspace` stated: the same call, except that it returns 1
+ * (hipErrorInvalidValue) without launching anything when the split the call resolves to needs more than
+ * `workspace_bytes`.  For callers that pass Split_K <= 0: between their SpMM_WorkspaceBytes(.., 0) and the call,
+ * the library's choice for the shape may have changed (SpMM_SplitK_TableSet/TableLoad, SPMM_SPLITK_TABLE read at
+ * first use), and SpMM_SplitK_API has no way to notice that the buffer is now too small.  The reference's call
+ * (csrc/SpMM_API.cuh:47-110) takes Split_K from its caller only and has no such case.
+ */
+int SpMM_SplitK_API_Sized(hipStream_t stream, const void* values, const uint64_t* bitmaps, const int* offsets,
+                          const void* X, void* C, int M, int N, int K, void* workspace, size_t workspace_bytes,
+                          int Split_K);
+
+/*
  * SpMM, reference call-site form: same argument order as the 14-argument
  * SpMM_SplitK_API_bitmap_v3 the reference's callers use
  * (kernel_benchmark/spmm_test.cu:375-388, third_party/ft_spinfer.patch:3736-3749),

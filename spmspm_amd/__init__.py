@@ -16,6 +16,7 @@ from .api import (  # noqa: F401
     NOALLOC_SCRATCH_BYTES,
     SpMM_SplitK_API,
     SpMM_SplitK_API_NoAlloc,
+    SpMM_SplitK_API_Sized,
     SpMM_SplitK_API_BiasAct,
     SpMM_WorkspaceBytesBiasAct,
     SpMM_SplitK_API_bitmap_v3,

@@ -40,6 +40,8 @@ def library():
     L = C.CDLL(_LIBPATH)
     L.SpMM_SplitK_API.restype = C.c_int
     L.SpMM_SplitK_API.argtypes = [C.c_void_p] * 6 + [C.c_int] * 3 + [C.c_void_p, C.c_int]
+    L.SpMM_SplitK_API_Sized.restype = C.c_int
+    L.SpMM_SplitK_API_Sized.argtypes = [C.c_void_p] * 6 + [C.c_int] * 3 + [C.c_void_p, C.c_size_t, C.c_int]
     L.SpMM_SplitK_API_bitmap_v3.restype = C.c_int
     L.SpMM_SplitK_API_bitmap_v3.argtypes = [C.c_void_p] * 9 + [C.c_int] * 3 + [C.c_void_p, C.c_int]
     L.SpMM_SplitK_Auto.restype = C.c_int
@@ -243,6 +245,13 @@ def SpMM_SplitK_API(stream, values, bitmaps, offsets, X, C_out, M, N, K, workspa
     """C = W*X on the device (include/spmm_api.h).  Tensors or raw device addresses.  Returns the hipError_t."""
     return library().SpMM_SplitK_API(_stream_handle(stream), _ptr(values), _ptr(bitmaps), _ptr(offsets), _ptr(X),
                                      _ptr(C_out), M, N, K, _ptr(workspace), Split_K)
+
+
+def SpMM_SplitK_API_Sized(stream, values, bitmaps, offsets, X, C_out, M, N, K, workspace, workspace_bytes, Split_K):
+    """SpMM_SplitK_API that refuses (returns 1) a workspace smaller than the split it resolves to needs."""
+    return library().SpMM_SplitK_API_Sized(_stream_handle(stream), _ptr(values), _ptr(bitmaps), _ptr(offsets),
+                                           _ptr(X), _ptr(C_out), M, N, K, _ptr(workspace), int(workspace_bytes),
+                                           Split_K)
 
 
 NOALLOC_SCRATCH_BYTES = 32 << 20  # SPMM_NOALLOC_SCRATCH_BYTES of include/spmm_api.h

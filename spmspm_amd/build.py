@@ -93,6 +93,38 @@ def build_stream_probe(verbose=False):
     return PROBE_PATH
 
 
+def kernel_resources(source, extra_flags=()):
+    """Compiles the device side of one source to assembly and returns, per kernel, the registers it uses and what
+    it spills: {mangled name: {"vgpr": n, "sgpr": n, "vgpr_spill": n, "sgpr_spill": n, "scratch_bytes": n}}.
+    A kernel that spills inside its tile loop loses a large factor without failing any numerical test."""
+    import re
+    import tempfile
+    fd, asm = tempfile.mkstemp(suffix=".s")
+    os.close(fd)
+    try:
+        cmd = [hipcc(), "-O3", "-std=c++17", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+               "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option", *extra_flags,
+               "-I", os.path.join(ROOT, "include"), "-I", CSRC, "--cuda-device-only", "-S",
+               os.path.join(CSRC, source), "-o", asm]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            sys.stderr.write(proc.stdout + proc.stderr)
+            raise RuntimeError("hipcc failed compiling " + source)
+        text = open(asm).read()
+    finally:
+        os.unlink(asm)
+    out = {}
+    keys = {"vgpr_count": "vgpr", "sgpr_count": "sgpr", "vgpr_spill_count": "vgpr_spill",
+            "sgpr_spill_count": "sgpr_spill", "private_segment_fixed_size": "scratch_bytes"}
+    for block in text.split("  - .agpr_count")[1:]:  # one entry of amdhsa.kernels each
+        name = re.search(r"^\s+\.name:\s+(\S+)", block, re.M)
+        if not name:
+            continue
+        out[name.group(1)] = {v: int(re.search(r"^\s+\.%s:\s+(\d+)" % k, block, re.M).group(1))
+                              for k, v in keys.items()}
+    return out
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
     print(build_variants_library(verbose=True))

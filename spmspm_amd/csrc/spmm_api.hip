@@ -323,6 +323,23 @@ extern "C" int SpMM_SplitK_API(hipStream_t stream, const void* values, const uin
     return run(stream, values, bitmaps, offsets, X, C, M, N, K, workspace, sk, /*fp32_partials=*/true);
 }
 
+extern "C" int SpMM_SplitK_API_Sized(hipStream_t stream, const void* values, const uint64_t* bitmaps,
+                                     const int* offsets, const void* X, void* C, int M, int N, int K, void* workspace,
+                                     size_t workspace_bytes, int Split_K)
+{
+    if (int e = check_shape(M, N, K))
+        return refuse(e);
+    // resolved once: the size check and the launch see the same split
+    const int sk = Split_K <= 0 ? split_k_for(M, N, K) : clamp_split_k(Split_K, K);
+    if (sk > 1 && sizeof(float) * (size_t)M * (size_t)N * (size_t)sk > workspace_bytes) {
+        std::printf("MM_Sparse_API Error: workspace of %zu bytes, Split_K %d needs %zu!\n", workspace_bytes, sk,
+                    sizeof(float) * (size_t)M * (size_t)N * (size_t)sk);
+        std::fflush(stdout);
+        return refuse((int)hipErrorInvalidValue);
+    }
+    return run(stream, values, bitmaps, offsets, X, C, M, N, K, workspace, sk, /*fp32_partials=*/true);
+}
+
 extern "C" size_t SpMM_WorkspaceBytesBiasAct(int M, int N, int K, int Split_K)
 {
     if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)

@@ -22,7 +22,7 @@ def test_header_declares_the_expected_entry_points():
               "Our_GenSparseMatrixBinFile", "SpMM_SplitK_Auto", "SpMM_WorkspaceBytes", "SpMM_Version", "SpMM_TimeNextCall",
               "SpMM_SplitK_API_BiasAct", "SpMM_WorkspaceBytesBiasAct", "SpMM_EncodeDevice_Bitmaps",
               "SpMM_EncodeDevice_Values", "SpMM_SplitK_TableSet", "SpMM_SplitK_TableLoad", "SpMM_SplitK_TableSave",
-              "SpMM_SplitK_TableClear", "SpMM_SplitK_API_NoAlloc"):
+              "SpMM_SplitK_TableClear", "SpMM_SplitK_API_NoAlloc", "SpMM_SplitK_API_Sized"):
         assert n in names
 
 
@@ -132,3 +132,29 @@ def test_tuner_candidates_and_presets():
     assert tuner.candidate_splits(5120) == list(range(1, 13))
     assert tuner.candidate_splits(256) == [1] and tuner.candidate_splits(512) == [1, 2]
     assert (28672, 7168) in tuner.PRESETS["opt30b"] and len(tuner.PRESETS["opt13b"]) == 4
+
+
+def test_sized_entry_point_refuses_a_small_workspace_without_a_gpu(capfd):
+    """The size check comes before anything touches the device: a too-small workspace returns
+    hipErrorInvalidValue for an explicit split and for the library's own choice, also after the table has changed
+    that choice behind the caller's back."""
+    M, N, K = 4096, 16, 4096
+    need4 = S.SpMM_WorkspaceBytes(M, N, K, 4)
+
+    def call(m, n, k, ws_bytes, sk):  # raw C call: null stream and null pointers, nothing is launched
+        return S.library().SpMM_SplitK_API_Sized(None, None, None, None, None, None, m, n, k, None, ws_bytes, sk)
+
+    assert call(M, N, K, need4 - 1, 4) == 1
+    assert "workspace" in capfd.readouterr().out
+    S.SpMM_SplitK_TableClear()
+    try:
+        small = S.SpMM_WorkspaceBytes(M, N, K, 0)
+        sk0 = S.SpMM_SplitK_Auto(M, N, K)
+        S.SpMM_SplitK_TableSet(M, N, K, sk0 + 3)           # the choice grows after the buffer was sized
+        assert S.SpMM_WorkspaceBytes(M, N, K, 0) > small
+        assert call(M, N, K, small, 0) == 1
+    finally:
+        S.SpMM_SplitK_TableClear()
+    # shape errors keep their own codes
+    assert call(M, 24, K, 1 << 30, 1) == 999
+    assert call(M + 1, N, K, 1 << 30, 1) == 1

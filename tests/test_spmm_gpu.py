@@ -326,6 +326,31 @@ def test_library_split_needs_workspace(torch, capfd):
     assert "workspace" in capfd.readouterr().out
 
 
+def test_sized_entry_point_matches_and_refuses(torch, oracle, capfd):
+    """SpMM_SplitK_API_Sized: the same result as SpMM_SplitK_API bit for bit with a workspace that is large enough,
+    C untouched and hipErrorInvalidValue with one that is a byte short (explicit and automatic split)."""
+    M, K, N = 512, 2048, 16
+    W = make_weight(M, K, 0.6, seed=11)
+    X = make_activations(K, N, seed=12)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    d = Device(torch, comp)
+    x = torch.from_numpy(X.view(np.int16).copy()).to("cuda:0")
+    for sk in (0, 3):
+        need = S.SpMM_WorkspaceBytes(M, N, K, sk)
+        assert need > 0
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda:0")
+        out = torch.full((N, M), 0x7e00, dtype=torch.int16, device="cuda:0")
+        assert S.SpMM_SplitK_API_Sized(None, d.values, d.bitmaps, d.offsets, x, out, M, N, K, ws, need, sk) == 0
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy().view(np.uint16), d.spmm(X, sk).view(np.uint16))
+        out.fill_(0x7e00)
+        assert S.SpMM_SplitK_API_Sized(None, d.values, d.bitmaps, d.offsets, x, out, M, N, K, ws, need - 1,
+                                       sk) == S.api.HIP_ERROR_INVALID_VALUE
+        torch.cuda.synchronize()
+        assert (out == 0x7e00).all()
+    assert "workspace" in capfd.readouterr().out
+
+
 def test_linearity_at_full_size(torch):
     """OPT-13B QKV shape: C(X1 + X2) == C(X1) + C(X2) within the contract, and C(0) == 0."""
     M, K, N = 15360, 5120, 16
