@@ -421,12 +421,7 @@ def main():
 
     # HBM bytes per launch of the main kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE.  The record
     # is only quoted when it was taken for exactly what ran here: same workload, width, sparsity, Split_K, kernel.
-    # (the dispatch of spmm::launch_spmm: the wide kernel for N a multiple of 128 on at least 256 rows)
-    if N % 128 == 0 and M >= 256:
-        kernel_name = f"spmm::spmm_bitmap_wide<8, {'true' if split_k > 1 else 'false'}>"
-    else:
-        nt = 1 if N <= 16 else (2 if N == 32 else 4)
-        kernel_name = f"spmm::spmm_bitmap_rows<{nt}, {'true' if split_k > 1 else 'false'}>"
+    kernel_name = L.SpMM_KernelName(M, N, K, split_k).decode()
     traffic, traffic_note = None, "no record for this configuration in profiles/traffic.json"
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):

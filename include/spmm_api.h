@@ -223,6 +223,15 @@ void Our_GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int K, char* C
  */
 void SpMM_TimeNextCall(hipEvent_t before_main, hipEvent_t after_main);
 
+/*
+ * Name of the main kernel a call with these dimensions dispatches, as a profiler prints it, e.g.
+ * "spmm::spmm_bitmap_rows<1, true>" (second template argument: fp32 partial sums to the workspace).  Split_K <= 0
+ * asks for the library's own split.  Reporting aid for benchmarks that key profiler records by kernel; no
+ * reference counterpart.  The string belongs to the library and is valid until the thread's next call of this
+ * function; NULL for dimensions the SpMM calls refuse.
+ */
+const char* SpMM_KernelName(int M, int N, int K, int Split_K);
+
 /* Library version string, e.g. "spmm-gfx950 0.1". */
 const char* SpMM_Version(void);
 

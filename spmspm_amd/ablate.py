@@ -191,8 +191,8 @@ def main(argv=None):
     from .synthetic import make_activations, make_weight
     M, K = (int(v) for v in a.shape.lower().split("x"))
     N = a.n
-    if N > 64 and N % 128 == 0:
-        ap.error("these patches are of spmm_bitmap_rows; N a multiple of 128 runs on the wide kernel")
+    if N >= 64 and M >= 256:
+        ap.error("these patches are of spmm_bitmap_rows; N >= 64 on at least 256 rows runs on the wide kernel")
     dev = torch.device("cuda:0")
     W = make_weight(M, K, a.sparsity, seed=0, pruning="random")
     comp = S.InitSparseMatrixA_bitmap(W)

@@ -72,6 +72,8 @@ def library():
     L.Our_GenSparseMatrixBinFile.restype = None
     L.Our_GenSparseMatrixBinFile.argtypes = [C.c_char_p, C.c_int, C.c_int] + [C.c_char_p] * 6
     L.SpMM_Version.restype = C.c_char_p
+    L.SpMM_KernelName.restype = C.c_char_p
+    L.SpMM_KernelName.argtypes = [C.c_int] * 4
     L.SpMM_TimeNextCall.restype = None
     L.SpMM_TimeNextCall.argtypes = [C.c_void_p, C.c_void_p]
     _lib = L

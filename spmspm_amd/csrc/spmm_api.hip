@@ -31,7 +31,7 @@ int clamp_split_k(int split_k, int K)
     return split_k < 1 ? 1 : split_k;
 }
 
-// K split of the wide kernel (N a multiple of 128, spmm_kernel_wide.hiph).  A workgroup covers 256 rows x 128 columns
+// K split of the wide kernel (N a multiple of 64, spmm_kernel_wide.hiph).  A workgroup covers 256 rows x 128 columns (64 at N = 64)
 // x one K batch and two workgroups fit a CU, so the 512 slots are the unit: one round of at most 512 workgroups,
 // each walking ceil(nkb / split) k blocks plus a start-up of about two.  Measured on OPT-66B FFN2 (9216 x 36864,
 // N = 128): a workgroup alone on its CU takes 2.2 us per k block, two sharing a CU 3.45 us each (ratio 1.57);
@@ -40,7 +40,7 @@ int clamp_split_k(int split_k, int K)
 int auto_split_k_wide(int M, int N, int K)
 {
     const int    nkb  = K / 64;
-    const long   base = (long)((M / 64 + 3) / 4) * (N / 128);
+    const long   base = (long)((M / 64 + 3) / 4) * (N / spmm::wide_tile_n(N));
     const double kSlots = 512.0, kAloneSlots = 256.0, kShared = 1.57, kStartup = 2.0;
     int          best = 1;
     double       best_c = 1e30;
@@ -465,6 +465,20 @@ extern "C" void SpMM_Debug_SetKernelVariant(int variant)
     spmm::kernel_variant() = variant;
 }
 #endif
+
+extern "C" const char* SpMM_KernelName(int M, int N, int K, int Split_K)
+{
+    if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
+        return nullptr;
+    thread_local char name[64];
+    const int         sk   = Split_K <= 0 ? split_k_for(M, N, K) : clamp_split_k(Split_K, K);
+    const char*       fp32 = sk > 1 ? "true" : "false"; // SpMM_SplitK_API: partial sums in fp32 whenever K is split
+    if (spmm::use_wide_kernel(M, N))
+        std::snprintf(name, sizeof name, "spmm::spmm_bitmap_wide<%d, %s>", spmm::wide_tile_n(N) / 16, fp32);
+    else
+        std::snprintf(name, sizeof name, "spmm::spmm_bitmap_rows<%d, %s>", spmm::tile_n(N) / 16, fp32);
+    return name;
+}
 
 extern "C" const char* SpMM_Version(void)
 {

@@ -22,7 +22,7 @@ def test_header_declares_the_expected_entry_points():
               "Our_GenSparseMatrixBinFile", "SpMM_SplitK_Auto", "SpMM_WorkspaceBytes", "SpMM_Version", "SpMM_TimeNextCall",
               "SpMM_SplitK_API_BiasAct", "SpMM_WorkspaceBytesBiasAct", "SpMM_EncodeDevice_Bitmaps",
               "SpMM_EncodeDevice_Values", "SpMM_SplitK_TableSet", "SpMM_SplitK_TableLoad", "SpMM_SplitK_TableSave",
-              "SpMM_SplitK_TableClear", "SpMM_SplitK_API_NoAlloc", "SpMM_SplitK_API_Sized"):
+              "SpMM_SplitK_TableClear", "SpMM_SplitK_API_NoAlloc", "SpMM_SplitK_API_Sized", "SpMM_KernelName"):
         assert n in names
 
 
@@ -165,3 +165,14 @@ def test_sized_entry_point_refuses_a_small_workspace_without_a_gpu(capfd):
     # shape errors keep their own codes
     assert call(M, 24, K, 1 << 30, 1) == 999
     assert call(M + 1, N, K, 1 << 30, 1) == 1
+
+
+def test_kernel_name_follows_the_dispatch():
+    name = lambda *a: (S.library().SpMM_KernelName(*a) or b"").decode()
+    assert name(28672, 16, 7168, 4) == "spmm::spmm_bitmap_rows<1, true>"
+    assert name(28672, 8, 7168, 1) == "spmm::spmm_bitmap_rows<1, false>"
+    assert name(28672, 32, 7168, 1) == "spmm::spmm_bitmap_rows<2, false>"
+    assert name(9216, 64, 36864, 14) == "spmm::spmm_bitmap_wide<4, true>"
+    assert name(128, 64, 4096, 2) == "spmm::spmm_bitmap_rows<4, true>"   # fewer than 256 rows
+    assert name(9216, 256, 36864, 7) == "spmm::spmm_bitmap_wide<8, true>"
+    assert name(9216, 24, 36864, 1) == "" and name(100, 16, 64, 1) == ""
