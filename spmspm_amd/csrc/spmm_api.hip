@@ -70,7 +70,7 @@ int auto_split_k_wide(int M, int N, int K)
 //   partials a split adds the reduction kernel, and every batch writes and re-reads an fp32 slab of M*N.
 int auto_split_k(int M, int N, int K)
 {
-    if (spmm::use_wide_kernel(M, N))
+    if (spmm::use_wide_kernel(M, N, K))
         return auto_split_k_wide(M, N, K);
     const int    nkb  = K / 64;
     const long   base = (long)(M / 64) * spmm::column_blocks(N);
@@ -473,7 +473,7 @@ extern "C" const char* SpMM_KernelName(int M, int N, int K, int Split_K)
     thread_local char name[64];
     const int         sk   = Split_K <= 0 ? split_k_for(M, N, K) : clamp_split_k(Split_K, K);
     const char*       fp32 = sk > 1 ? "true" : "false"; // SpMM_SplitK_API: partial sums in fp32 whenever K is split
-    if (spmm::use_wide_kernel(M, N))
+    if (spmm::use_wide_kernel(M, N, K))
         std::snprintf(name, sizeof name, "spmm::spmm_bitmap_wide<%d, %s>", spmm::wide_tile_n(N) / 16, fp32);
     else
         std::snprintf(name, sizeof name, "spmm::spmm_bitmap_rows<%d, %s>", spmm::tile_n(N) / 16, fp32);

@@ -173,6 +173,8 @@ def test_kernel_name_follows_the_dispatch():
     assert name(28672, 8, 7168, 1) == "spmm::spmm_bitmap_rows<1, false>"
     assert name(28672, 32, 7168, 1) == "spmm::spmm_bitmap_rows<2, false>"
     assert name(9216, 64, 36864, 14) == "spmm::spmm_bitmap_wide<4, true>"
+    assert name(28672, 64, 7168, 4) == "spmm::spmm_bitmap_wide<4, true>"
+    assert name(5120, 64, 5120, 3) == "spmm::spmm_bitmap_rows<4, true>"  # too few tiles for one round of long batches
     assert name(128, 64, 4096, 2) == "spmm::spmm_bitmap_rows<4, true>"   # fewer than 256 rows
     assert name(9216, 256, 36864, 7) == "spmm::spmm_bitmap_wide<8, true>"
     assert name(9216, 24, 36864, 1) == "" and name(100, 16, 64, 1) == ""
