@@ -32,13 +32,28 @@ class Device:
         self.median = torch.from_numpy(comp.median.copy() if comp.median.size else np.zeros(4, np.int32)).to(dev)
         self.max_nnz = torch.tensor([comp.max_nnz_rounded], dtype=torch.int32, device=dev)
 
-    def spmm(self, X, split_k, entry="api"):
+    def spmm(self, X, split_k, entry="api", lib=None):
+        """`lib`: a ctypes handle of another build of the library (the variants build) to call instead."""
         torch = self.torch
         N, K = X.shape
         M = self.c.M
         x = torch.from_numpy(X.view(np.int16).copy()).to("cuda:0")
         out = torch.full((N, M), 0x7e00, dtype=torch.int16, device="cuda:0")  # NaN-filled: C must be overwritten
-        if entry == "api":
+        if lib is not None:
+            stream = torch.cuda.current_stream().cuda_stream
+            sk = split_k if split_k > 0 else S.SpMM_SplitK_Auto(M, N, K)
+            if entry == "api":
+                ws = torch.empty(max(4 * M * N * sk, 16), dtype=torch.uint8, device="cuda:0")
+                err = lib.SpMM_SplitK_API(stream, self.values.data_ptr(), self.bitmaps.data_ptr(),
+                                          self.offsets.data_ptr(), x.data_ptr(), out.data_ptr(), M, N, K,
+                                          ws.data_ptr(), sk)
+            else:
+                ws = torch.empty(max(2 * M * N * sk, 16), dtype=torch.uint8, device="cuda:0")
+                err = lib.SpMM_SplitK_API_bitmap_v3(stream, None, self.values.data_ptr(), self.offsets.data_ptr(),
+                                                    self.median.data_ptr(), self.bitmaps.data_ptr(),
+                                                    self.max_nnz.data_ptr(), x.data_ptr(), out.data_ptr(), M, N, K,
+                                                    ws.data_ptr(), sk)
+        elif entry == "api":
             nbytes = S.SpMM_WorkspaceBytes(M, N, K, split_k)
             ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda:0") if nbytes else None
             err = S.SpMM_SplitK_API(None, self.values, self.bitmaps, self.offsets, x, out, M, N, K, ws, split_k)
@@ -49,6 +64,22 @@ class Device:
         assert err == 0, f"hipError_t {err}"
         torch.cuda.synchronize()
         return out.cpu().numpy().view(np.float16)
+
+
+@pytest.fixture(scope="module")
+def variants_lib():
+    """The test build of the library (libSpMM_API_variants.so): the same entry points plus SpMM_Debug_SetKernelVariant."""
+    import ctypes as C
+    path = os.path.join(os.path.dirname(S.library_path()), "libSpMM_API_variants.so")
+    assert os.path.exists(path), "build it with __graft_entry__.build()"
+    L = C.CDLL(path)
+    L.SpMM_SplitK_API.restype = C.c_int
+    L.SpMM_SplitK_API.argtypes = [C.c_void_p] * 6 + [C.c_int] * 3 + [C.c_void_p, C.c_int]
+    L.SpMM_SplitK_API_bitmap_v3.restype = C.c_int
+    L.SpMM_SplitK_API_bitmap_v3.argtypes = [C.c_void_p] * 9 + [C.c_int] * 3 + [C.c_void_p, C.c_int]
+    L.SpMM_Debug_SetKernelVariant.argtypes = [C.c_int]
+    yield L
+    L.SpMM_Debug_SetKernelVariant(2)
 
 
 def _oracle_C(oracle, comp, X, split_k=1, partial_fp16=False):
@@ -189,10 +220,12 @@ WIDE_CASES = [
 
 
 @pytest.mark.parametrize("M,K,N,density,splits", WIDE_CASES)
-def test_wide_kernel_exact_on_small_integers(torch, oracle, M, K, N, density, splits):
-    """N a multiple of 128 and M >= 256 run on the wide kernel (a group tile decoded once per 128 columns, X staged
-    in LDS per workgroup).  Bit-identical to the oracle where fp32 accumulation is exact: the library's own Split_K
-    and explicit ones, fp32 partial slabs ("api") and fp16 ones ("v3")."""
+def test_wide_kernel_exact_on_small_integers(torch, oracle, variants_lib, M, K, N, density, splits):
+    """The wide kernel (a group tile decoded once per 128 columns, X staged in LDS per workgroup) on shapes that
+    exercise its corners.  The shipped dispatch sends only large matrices to it, so these small ones are run through
+    the test build with the wide kernel forced, and once more through the shipped library (whatever kernel it picks).
+    Bit-identical to the oracle where fp32 accumulation is exact: the library's own Split_K and explicit ones, fp32
+    partial slabs ("api") and fp16 ones ("v3")."""
     rng = np.random.default_rng(M + K + N)
     W, X = _small_integer_problem(rng, M, K, N, density)
     W[64:128, :] = 0                      # an all-zero row block
@@ -200,11 +233,17 @@ def test_wide_kernel_exact_on_small_integers(torch, oracle, M, K, N, density, sp
     comp = S.InitSparseMatrixA_bitmap(W)
     dev = Device(torch, comp)
     want = _oracle_C(oracle, comp, X).view(np.uint16)
-    for sk in (0,) + tuple(splits):
-        print(f"case wide M={M} K={K} N={N} density={density} sk={sk}", flush=True)
-        assert np.array_equal(dev.spmm(X, sk, "api").view(np.uint16), want), ("api", sk)
-    for sk in splits[:2]:
-        assert np.array_equal(dev.spmm(X, sk, "v3").view(np.uint16), want), ("v3", sk)
+    variants_lib.SpMM_Debug_SetKernelVariant(4)
+    try:
+        for sk in (0,) + tuple(splits):
+            print(f"case wide M={M} K={K} N={N} density={density} sk={sk}", flush=True)
+            assert np.array_equal(dev.spmm(X, sk, "api", lib=variants_lib).view(np.uint16), want), ("api", sk)
+        for sk in splits[:2]:
+            assert np.array_equal(dev.spmm(X, sk, "v3", lib=variants_lib).view(np.uint16), want), ("v3", sk)
+    finally:
+        variants_lib.SpMM_Debug_SetKernelVariant(2)
+    for sk in (0, splits[-1]):
+        assert np.array_equal(dev.spmm(X, sk, "api").view(np.uint16), want), ("shipped dispatch", sk)
 
 
 def test_golden_fixtures_decode_on_device(torch, golden):
