@@ -26,9 +26,13 @@ PRESETS = {
 }
 
 
-def candidate_splits(K, limit=12):
-    """1..limit, never more batches than a quarter of the group-tile columns (one tile per wave and batch)."""
+def candidate_splits(K, limit=12, M=None, N=None):
+    """1..limit, never more batches than a quarter of the group-tile columns (one tile per wave and batch).  With M
+    and N given and the shape dispatched to the wide kernel (four row blocks per workgroup, so its good splits are
+    larger): 1..32, never more than half of the group-tile columns."""
     nkb = K // 64
+    if M is not None and N is not None and b"wide" in (A.library().SpMM_KernelName(M, N, K, 1) or b""):
+        return [s for s in range(1, 33) if s <= max(1, nkb // 2)]
     return [s for s in range(1, limit + 1) if s <= max(1, nkb // 4)]
 
 
@@ -64,7 +68,7 @@ def tune_shape(M, N, K, sparsity=0.6, candidates=None, device="cuda:0", iters=30
     layers = [first] + [first.clone() for _ in range(n_copies - 1)]
     x = torch.from_numpy(make_activations(K, N, seed=seed).view(np.int16).copy()).to(device).view(torch.float16)
     times = {}
-    cands = list(candidates or candidate_splits(K))
+    cands = list(candidates or candidate_splits(K, M=M, N=N))
     time_split_k(layers, x, cands[0], iters=max(iters, 300))  # not kept: the first calls after idle run at ramping clocks
     for sk in cands:
         times[sk] = time_split_k(layers, x, sk, iters=iters)
