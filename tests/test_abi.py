@@ -178,3 +178,10 @@ def test_kernel_name_follows_the_dispatch():
     assert name(128, 64, 4096, 2) == "spmm::spmm_bitmap_rows<4, true>"   # fewer than 256 rows
     assert name(9216, 256, 36864, 7) == "spmm::spmm_bitmap_wide<8, true>"
     assert name(9216, 24, 36864, 1) == "" and name(100, 16, 64, 1) == ""
+
+
+def test_row_count_limit_is_reported(capfd):
+    """Row blocks are the z dimension of the launch grid: more than 65535 of them is refused before any launch."""
+    L = S.library()
+    assert L.SpMM_SplitK_API(None, None, None, None, None, None, 64 * 65536, 16, 64, None, 1) == 1
+    assert "65535" in capfd.readouterr().out
