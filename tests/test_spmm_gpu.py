@@ -719,6 +719,39 @@ def test_seeded_random_shapes(torch, oracle):
             assert_spmm_close(dev.spmm(X, sk, "v3"), _oracle_C(oracle, comp, X, sk_eff, True), f"case {case} v3")
 
 
+def test_randomized_exact_on_every_dispatch(torch, variants_lib):
+    """Eighty seeded random problems in small integers (exact in fp32, so the product is known bit for bit from a
+    float64 product) through the shipped dispatch, the row-per-lane kernel everywhere and the wide kernel everywhere:
+    up to 2048 rows and 4096 columns, every supported width up to 384 columns, a different density for every group
+    tile of a matrix (empty, nearly empty, ..., full side by side), the library's own split, no split, and two
+    random ones of which one may exceed the number of k blocks (the library then uses one batch per k block)."""
+    rng = np.random.default_rng(31)
+    stream = torch.cuda.current_stream().cuda_stream
+    try:
+        for case in range(80):
+            M = 64 * int(rng.integers(1, 33))
+            K = 64 * int(rng.integers(1, 65))
+            N = int(rng.choice([8, 16, 32, 64, 128, 256, 384]))
+            dens = rng.choice([0.0, 0.02, 0.3, 0.5, 0.8, 1.0], size=(M // 64, K // 64), p=[0.1, 0.1, 0.4, 0.2, 0.1, 0.1])
+            W = rng.integers(-2, 3, (M, K)).astype(np.float16)
+            W[rng.random((M, K)) >= np.kron(dens, np.ones((64, 64)))] = 0
+            X = rng.integers(-2, 3, (N, K)).astype(np.float16)
+            want = (X.astype(np.float64) @ W.astype(np.float64).T).astype(np.float16).view(np.uint16)
+            dev = Device(torch, S.InitSparseMatrixA_bitmap(W))
+            nkb = K // 64
+            splits = sorted({0, 1, int(rng.integers(1, nkb + 1)), int(rng.integers(1, nkb + 4))})
+            print(f"case {case}: M={M} K={K} N={N} splits={splits}", flush=True)
+            for variant in (2, 3, 4):
+                if variant == 4 and (N % 64 != 0 or M < 256):
+                    continue
+                variants_lib.SpMM_Debug_SetKernelVariant(variant)
+                for sk in splits:
+                    got = dev.spmm(X, sk, "api", lib=variants_lib).view(np.uint16)
+                    assert np.array_equal(got, want), (case, M, K, N, variant, sk)
+    finally:
+        variants_lib.SpMM_Debug_SetKernelVariant(2)
+
+
 @pytest.mark.parametrize("args", [(1024, 1024, 16, 70, 2), (2048, 512, 8, 50, 1), (512, 4096, 32, 60, 4),
                                   (1024, 2048, 64, 40, 3), (256, 1024, 128, 90, 2)])
 def test_cpp_caller_of_the_library(args):
