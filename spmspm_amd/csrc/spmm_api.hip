@@ -36,12 +36,15 @@ int clamp_split_k(int split_k, int K)
 // each walking ceil(nkb / split) k blocks plus a start-up of about two.  Measured on OPT-66B FFN2 (9216 x 36864,
 // N = 128): a workgroup alone on its CU takes 2.2 us per k block, two sharing a CU 3.45 us each (ratio 1.57);
 // Split_K 7 / 12 / 14 / 16 -> 252 / 432 / 504 / 576 workgroups -> 177 / 151 / 141 / 177 us.  The partial slabs of a
-// split are re-read from cache by the reduction, which adds little.
+// split are re-read from cache by the reduction, which adds little.  Over the 20 shapes on which the wide kernel was
+// timed at every Split_K up to 32 (OPT-13B, 30B and 66B linears at N = 64 and 128) a sharing ratio of 1.4 and a
+// tenth added to a launch that needs a second round pick the measured best split on all of them; with 1.57 and no
+// addition three were off by 3 to 8 %.
 int auto_split_k_wide(int M, int N, int K)
 {
     const int    nkb  = K / 64;
     const long   base = (long)((M / 64 + 3) / 4) * (N / spmm::wide_tile_n(N));
-    const double kSlots = 512.0, kAloneSlots = 256.0, kShared = 1.57, kStartup = 2.0;
+    const double kSlots = 512.0, kAloneSlots = 256.0, kShared = 1.4, kSecondRound = 1.1, kStartup = 2.0;
     int          best = 1;
     double       best_c = 1e30;
     int          max_sk = nkb / 2 > 0 ? nkb / 2 : 1; // at least two k blocks per batch
@@ -51,7 +54,7 @@ int auto_split_k_wide(int M, int N, int K)
         const double wgs    = (double)base * sk;
         const double rounds = (double)((long)((wgs + kSlots - 1) / kSlots));
         const double steps  = (double)((nkb + sk - 1) / sk) + kStartup;
-        double       cost   = rounds * steps * (wgs > kAloneSlots ? kShared : 1.0);
+        double       cost   = rounds * steps * (wgs > kAloneSlots ? kShared : 1.0) * (rounds > 1.0 ? kSecondRound : 1.0);
         if (sk > 1)
             cost += 1.0 + sk * ((double)M * N * 8.0) / 8e12 / 2.2e-6;
         if (cost < best_c - 1e-9) {

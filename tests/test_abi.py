@@ -99,15 +99,17 @@ def test_split_table_overrides_the_cost_model_and_round_trips_through_a_file(tmp
 
 
 def test_shipped_split_table_loads_and_covers_the_decode_widths():
-    """The measured table in spmspm_amd/tuned/ parses, lists the OPT-13B and OPT-30B linears at N = 8, 16, 32 and
-    64, and takes precedence over the cost model once loaded."""
+    """The measured table in spmspm_amd/tuned/ parses, lists the OPT-13B, OPT-30B and OPT-66B linears at N = 8, 16,
+    32, 64 and 128, and takes precedence over the cost model once loaded."""
     path = os.path.join(ROOT, "spmspm_amd", "tuned", "splitk_mi355x_s60.txt")
     try:
-        assert S.SpMM_SplitK_TableLoad(path) == 33
+        assert S.SpMM_SplitK_TableLoad(path) == 60
         for M, K in [(15360, 5120), (5120, 5120), (20480, 5120), (5120, 20480), (28672, 7168), (7168, 7168),
-                     (21504, 7168), (7168, 28672)]:
+                     (21504, 7168), (7168, 28672), (27648, 9216), (9216, 9216), (36864, 9216), (9216, 36864)]:
             for N in (8, 16, 32):
                 assert 1 <= S.SpMM_SplitK_Auto(M, N, K) <= 12
+            for N in (64, 128):
+                assert 1 <= S.SpMM_SplitK_Auto(M, N, K) <= 32
         table = {}
         for line in open(path):
             if line.strip() and not line.startswith("#"):
