@@ -421,6 +421,22 @@ def test_target_shape_against_oracle(torch, oracle):
     assert_spmm_close(dev.spmm(X, 4, "v3"), want, "target v3 sk=4")
 
 
+def test_cpu_reference_configuration_on_the_device(torch, oracle):
+    """The configuration the reference runs on a CPU alone (4096x4096, 50 % random unstructured, N = 16, seed 0):
+    the whole output against the oracle, with the library's split, unsplit, and through the 14-argument entry."""
+    from spmspm_amd.synthetic import WORKLOADS
+    w = WORKLOADS["cpu_plumbing_4096"]
+    M, K, N = w["M"], w["K"], w["N"]
+    W = make_weight(M, K, w["sparsity"], seed=0, pruning=w["pruning"])
+    X = make_activations(K, N, seed=0)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    dev = Device(torch, comp)
+    want = _oracle_C(oracle, comp, X)
+    for sk in (0, 1):
+        assert_spmm_close(dev.spmm(X, sk), want, f"4096x4096 sk={sk}")
+    assert_spmm_close(dev.spmm(X, 3, "v3"), _oracle_C(oracle, comp, X, 3, True), "4096x4096 v3 sk=3")
+
+
 @pytest.mark.parametrize("sparsity", [0.4, 0.5])
 def test_opt30b_ffn1_full_size_other_batches_and_sparsities(torch, sparsity):
     """OPT-30B FFN1 28672x7168 at the denser settings of the benchmark set, N = 8 and 32, magnitude pruning:
