@@ -102,6 +102,8 @@ int SpMM_SplitK_API_bitmap_v3(hipStream_t stream, const void* A, const void* Com
  * (end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:23).
  */
 int SpMM_SplitK_Auto(int M, int N, int K);
+/* The built-in cost model's choice for the shape, whatever the table of measured choices (below) holds. */
+int SpMM_SplitK_CostModel(int M, int N, int K);
 
 /*
  * Measured Split_K choices, which SpMM_SplitK_Auto (and every call with Split_K <= 0) prefers to its built-in
@@ -109,14 +111,20 @@ int SpMM_SplitK_Auto(int M, int N, int K);
  * (end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:23, keyed by M alone) and the SPLIT_K array of
  * kernel_benchmark/run_all_main.sh:5.  The table is keyed by (M, N, K) and shared by all threads of the process.
  *   TableSet    records one choice; returns 0, or hipErrorInvalidValue for a shape the library does not run.
+ *   TableSetMany records `count` choices at once, `entries` holding {M, N, K, Split_K} four ints each (one copy of
+ *               the table instead of one per entry); returns 0, or hipErrorInvalidValue, recording nothing, when
+ *               any entry is one TableSet would refuse.
  *   TableLoad   adds the entries of a text file of "M N K Split_K" lines ('#' starts a comment); returns their
  *               number, -1 if the file cannot be opened, -2 on a malformed line.
  *   TableSave   writes the table in that format; returns the number of entries, -1 if the file cannot be written.
  *   TableClear  empties the table.
- * A file named by SPMM_SPLITK_TABLE in the environment is loaded the first time a choice is needed.
+ * The first time a choice is needed a file is loaded: the one SPMM_SPLITK_TABLE names in the environment, or, when
+ * that variable is not set, the measured table shipped with the library (tuned/splitk_mi355x.txt beside the
+ * library's directory) if it is there.  SPMM_SPLITK_TABLE set to an empty string loads nothing (cost model only).
  * A workspace must be sized (SpMM_WorkspaceBytes) after the table is in its final state.
  */
 int  SpMM_SplitK_TableSet(int M, int N, int K, int Split_K);
+int  SpMM_SplitK_TableSetMany(const int* entries, int count);
 int  SpMM_SplitK_TableLoad(const char* path);
 int  SpMM_SplitK_TableSave(const char* path);
 void SpMM_SplitK_TableClear(void);
@@ -147,9 +155,11 @@ size_t SpMM_WorkspaceBytesBiasAct(int M, int N, int K, int Split_K);
  * reference; it is for callers that cannot allocate device memory: code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc.  The fp32 partial sums of a split K go to a device array of
  * SPMM_NOALLOC_SCRATCH_BYTES that the library itself holds on every GPU it runs on until the process ends.
- * Arguments, Split_K <= 0 and results are those of SpMM_SplitK_API (the same kernels run); a call whose partial
+ * Arguments and results are those of SpMM_SplitK_API (the same kernels run).  An explicit Split_K whose partial
  * sums (4*M*N*Split_K bytes for Split_K > 1) exceed the array prints a message and returns 1
- * (hipErrorInvalidValue) without launching anything.  The call makes no hipMalloc/hipFree; the first call on a
+ * (hipErrorInvalidValue) without launching anything.  With Split_K <= 0 the library's own choice gives way to the
+ * largest split whose partial sums fit (an unsplit K needs none, so such a call always runs);
+ * SpMM_SplitK_AutoNoAlloc reports that split.  The call makes no hipMalloc/hipFree; the first call on a
  * device looks up the array's device address once (make that call outside a graph capture).
  * All calls on one GPU share the array: calls that overlap in time on one GPU (different streams, or graphs
  * replayed concurrently) race on it and must be serialised by the caller.
@@ -157,6 +167,7 @@ size_t SpMM_WorkspaceBytesBiasAct(int M, int N, int K, int Split_K);
 #define SPMM_NOALLOC_SCRATCH_BYTES (32u << 20)
 int SpMM_SplitK_API_NoAlloc(hipStream_t stream, const void* values, const uint64_t* bitmaps, const int* offsets,
                             const void* X, void* C, int M, int N, int K, int Split_K);
+int SpMM_SplitK_AutoNoAlloc(int M, int N, int K);
 
 /*
  * Host encoder, C twin of InitSparseMatrixA_bitmap
@@ -213,6 +224,34 @@ void Our_GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int K, char* C
                                 char* bitmapFileName, char* max_nnz_intileFileName, char* OutputSizesFileName);
 
 /*
+ * Readers of the six files Our_GenSparseMatrixBinFile writes: the consumer side, which in the reference is the
+ * FasterTransformer layer-weight loader (third_party/ft_spinfer.patch:2335-2357: loadDataArrayFromBin of
+ * .NZWeights/.gtile/.mtile/.ltile/.intile into device arrays sized from the model's configuration).
+ *   SpMM_ReadWeightFiles  reads them into malloc'd host arrays (free() each): values (val_count halves),
+ *                         TileOffsets_global (G+1 ints), TileOffsets_median (4G ints), bitmap (64G uint64) and the
+ *                         max-nnz hint.  TileOffsets_median, max_nnz_intile and val_count may be NULL.
+ *   SpMM_LoadWeightFiles  reads them and leaves them in device memory of the current device (hipMalloc +
+ *                         synchronous copies), ready to be passed to the SpMM entry points; median_d, max_nnz_d
+ *                         and val_count may be NULL (then those are not kept).  Release with SpMM_FreeWeights.
+ * Both check the sizes file against M and K ({val_count, G+1, 4G, 64G}, csrc/SpMM_API.cuh:304-308), every file's
+ * length and that the offsets start at 0, end at val_count and grow by multiples of 8 of at most 4096.
+ * Return G = (M/64)*(K/64), or -1 a file is missing or has another length, -2 the files do not match M and K or
+ * each other, -4 a required argument is NULL, -5 (Load only) a HIP call failed; nothing is returned or kept then.
+ * Unlike the reference's loader they never end the process.
+ */
+int  SpMM_ReadWeightFiles(const char* Compressed_ValFileName, const char* TileOffsets_globalFileName,
+                          const char* TileOffsets_medianFileName, const char* bitmapFileName,
+                          const char* max_nnz_intileFileName, const char* OutputSizesFileName, int M, int K,
+                          uint16_t** Compressed_Val, int** TileOffsets_global, int** TileOffsets_median,
+                          uint64_t** bitmap, int* max_nnz_intile, int* val_count);
+int  SpMM_LoadWeightFiles(const char* Compressed_ValFileName, const char* TileOffsets_globalFileName,
+                          const char* TileOffsets_medianFileName, const char* bitmapFileName,
+                          const char* max_nnz_intileFileName, const char* OutputSizesFileName, int M, int K,
+                          void** values_d, int** offsets_d, int** median_d, uint64_t** bitmaps_d, int** max_nnz_d,
+                          int* val_count);
+void SpMM_FreeWeights(void* values_d, int* offsets_d, int* median_d, uint64_t* bitmaps_d, int* max_nnz_d);
+
+/*
  * Timing aid with no counterpart in the reference (its harness times whole
  * calls with cudaEvents, kernel_benchmark/spmm_test.cu:374-411): the next SpMM
  * call made by this thread attaches the two events to the dispatch of its main
@@ -224,9 +263,11 @@ void Our_GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int K, char* C
 void SpMM_TimeNextCall(hipEvent_t before_main, hipEvent_t after_main);
 
 /*
- * Name of the main kernel a call with these dimensions dispatches, as a profiler prints it, e.g.
- * "spmm::spmm_bitmap_rows<1, true>" (second template argument: fp32 partial sums to the workspace).  Split_K <= 0
- * asks for the library's own split.  Reporting aid for benchmarks that key profiler records by kernel; no
+ * Name of the main kernel a call of SpMM_SplitK_API, SpMM_SplitK_API_Sized or SpMM_SplitK_API_NoAlloc with these
+ * dimensions dispatches, as a profiler prints it, e.g. "spmm::spmm_bitmap_rows<1, true>" (second template argument:
+ * fp32 partial sums to the workspace, which these three entry points use whenever K is split).  It does not hold
+ * for SpMM_SplitK_API_bitmap_v3 (fp16 partial sums: "false" for every split) or SpMM_SplitK_API_BiasAct (one fp32
+ * slab even for an unsplit K: "true" for every split).  Split_K <= 0 asks for the library's own split.  Reporting aid for benchmarks that key profiler records by kernel; no
  * reference counterpart.  The string belongs to the library and is valid until the thread's next call of this
  * function; NULL for dimensions the SpMM calls refuse.
  */

@@ -20,7 +20,11 @@ from .api import (  # noqa: F401
     SpMM_SplitK_API_BiasAct,
     SpMM_WorkspaceBytesBiasAct,
     SpMM_SplitK_API_bitmap_v3,
+    SpMM_ReadWeightFiles,
     SpMM_SplitK_Auto,
+    SpMM_SplitK_AutoNoAlloc,
+    SpMM_SplitK_CostModel,
+    SpMM_SplitK_TableSetMany,
     SpMM_SplitK_TableClear,
     SpMM_SplitK_TableLoad,
     SpMM_SplitK_TableSave,

@@ -48,6 +48,19 @@ def library():
     L.SpMM_SplitK_Auto.argtypes = [C.c_int] * 3
     L.SpMM_SplitK_TableSet.restype = C.c_int
     L.SpMM_SplitK_TableSet.argtypes = [C.c_int] * 4
+    L.SpMM_SplitK_CostModel.restype = C.c_int
+    L.SpMM_SplitK_CostModel.argtypes = [C.c_int] * 3
+    L.SpMM_SplitK_AutoNoAlloc.restype = C.c_int
+    L.SpMM_SplitK_AutoNoAlloc.argtypes = [C.c_int] * 3
+    L.SpMM_SplitK_TableSetMany.restype = C.c_int
+    L.SpMM_SplitK_TableSetMany.argtypes = [_i32p, C.c_int]
+    L.SpMM_ReadWeightFiles.restype = C.c_int
+    L.SpMM_ReadWeightFiles.argtypes = [C.c_char_p] * 6 + [C.c_int, C.c_int, C.POINTER(_u16p), C.POINTER(_i32p),
+                                                         C.POINTER(_i32p), C.POINTER(_u64p), _i32p, _i32p]
+    L.SpMM_LoadWeightFiles.restype = C.c_int
+    L.SpMM_LoadWeightFiles.argtypes = [C.c_char_p] * 6 + [C.c_int, C.c_int] + [C.POINTER(C.c_void_p)] * 5 + [_i32p]
+    L.SpMM_FreeWeights.restype = None
+    L.SpMM_FreeWeights.argtypes = [C.c_void_p] * 5
     L.SpMM_SplitK_TableLoad.restype = C.c_int
     L.SpMM_SplitK_TableLoad.argtypes = [C.c_char_p]
     L.SpMM_SplitK_TableSave.restype = C.c_int
@@ -162,6 +175,32 @@ def Our_GenSparseMatrixBinFile(dense_path, M, K, values_path, global_path, media
     library().Our_GenSparseMatrixBinFile(enc[0], M, K, *enc[1:])
 
 
+def SpMM_ReadWeightFiles(values_path, global_path, median_path, bitmap_path, max_nnz_path, sizes_path, M, K):
+    """The library's own reader of the six files (include/spmm_api.h) -> CompressedMatrix (per-tile counts from the
+    bitmaps).  Raises OSError / ValueError on the library's -1 / -2."""
+    enc = [os.fsencode(p) for p in (values_path, global_path, median_path, bitmap_path, max_nnz_path, sizes_path)]
+    vals, glo, med, bmp = _u16p(), _i32p(), _i32p(), _u64p()
+    mx, cnt = C.c_int(0), C.c_int(0)
+    G = library().SpMM_ReadWeightFiles(*enc, M, K, C.byref(vals), C.byref(glo), C.byref(med), C.byref(bmp),
+                                       C.byref(mx), C.byref(cnt))
+    if G == -1:
+        raise OSError("SpMM_ReadWeightFiles: a file is missing or has another length than the sizes file states")
+    if G < 0:
+        raise ValueError(f"SpMM_ReadWeightFiles: the files do not match M, K or each other ({G})")
+    n = cnt.value
+    bitmaps = np.ctypeslib.as_array(bmp, shape=(max(64 * G, 1),))[:64 * G].copy()
+    out = CompressedMatrix(
+        M=M, K=K, num_gtiles=G,
+        values=np.ctypeslib.as_array(vals, shape=(max(n, 1),))[:n].copy(),
+        tile_counts=_popcount64(bitmaps),
+        median=np.ctypeslib.as_array(med, shape=(max(4 * G, 1),))[:4 * G].copy(),
+        offsets=np.ctypeslib.as_array(glo, shape=(G + 1,)).copy(),
+        bitmaps=bitmaps, max_nnz=mx.value)
+    for p in (vals, glo, med, bmp):
+        _libc.free(C.cast(p, C.c_void_p))
+    return out
+
+
 def load_weight_files(values_path, global_path, median_path, bitmap_path, max_nnz_path, sizes_path, M, K):
     """Read the six files back (layout of csrc/SpMM_API.cuh:304-319) into a CompressedMatrix."""
     sizes = np.fromfile(sizes_path, dtype=np.int32)
@@ -201,6 +240,24 @@ def SpMM_SplitK_TableSet(M, N, K, Split_K):
     rc = library().SpMM_SplitK_TableSet(M, N, K, Split_K)
     if rc != 0:
         raise ValueError(f"SpMM_SplitK_TableSet({M}, {N}, {K}, {Split_K}) -> {rc}")
+
+
+def SpMM_SplitK_TableSetMany(entries):
+    """Record several measured choices at once: an iterable of (M, N, K, Split_K)."""
+    flat = np.ascontiguousarray(np.asarray(list(entries), dtype=np.int32).reshape(-1, 4))
+    rc = library().SpMM_SplitK_TableSetMany(flat.ctypes.data_as(_i32p), flat.shape[0])
+    if rc != 0:
+        raise ValueError(f"SpMM_SplitK_TableSetMany refused its entries ({rc})")
+
+
+def SpMM_SplitK_CostModel(M, N, K):
+    """The built-in cost model's Split_K for a shape, whatever the table holds."""
+    return library().SpMM_SplitK_CostModel(M, N, K)
+
+
+def SpMM_SplitK_AutoNoAlloc(M, N, K):
+    """The split SpMM_SplitK_API_NoAlloc uses for Split_K <= 0: the library's choice, held to what its array fits."""
+    return library().SpMM_SplitK_AutoNoAlloc(M, N, K)
 
 
 def SpMM_SplitK_TableLoad(path):

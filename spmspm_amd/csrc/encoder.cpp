@@ -278,3 +278,81 @@ extern "C" void Our_GenSparseMatrixBinFile(char* DenseMatrixFileName, int M, int
     f_nnz.write(reinterpret_cast<char*>(&max_nnz), sizeof(int));
     std::free(vals), std::free(cnt), std::free(median), std::free(global), std::free(bitmap);
 }
+
+// Reader of those six files (the consumer side: third_party/ft_spinfer.patch:2335-2357 loads them with
+// loadDataArrayFromBin into arrays sized from the model's configuration).  Unlike the writer it reports failure to
+// its caller instead of ending the process.
+namespace {
+
+// the whole file as `count` elements of `size` bytes, malloc'd; nullptr when it is missing or has another length
+void* read_exact(const char* path, size_t size, size_t count)
+{
+    std::FILE* f = std::fopen(path, "rb");
+    if (!f)
+        return nullptr;
+    void*  buf = std::malloc(size * count ? size * count : 1);
+    size_t got = buf ? std::fread(buf, size, count, f) : 0;
+    char   extra;
+    const bool longer = std::fread(&extra, 1, 1, f) == 1;
+    std::fclose(f);
+    if (buf == nullptr || got != count || longer) {
+        std::free(buf);
+        return nullptr;
+    }
+    return buf;
+}
+
+} // namespace
+
+extern "C" int SpMM_ReadWeightFiles(const char* Compressed_ValFileName, const char* TileOffsets_globalFileName,
+                                    const char* TileOffsets_medianFileName, const char* bitmapFileName,
+                                    const char* max_nnz_intileFileName, const char* OutputSizesFileName, int M, int K,
+                                    uint16_t** Compressed_Val, int** TileOffsets_global, int** TileOffsets_median,
+                                    uint64_t** bitmap, int* max_nnz_intile, int* val_count)
+{
+    if (!Compressed_ValFileName || !TileOffsets_globalFileName || !TileOffsets_medianFileName || !bitmapFileName ||
+        !max_nnz_intileFileName || !OutputSizesFileName || !Compressed_Val || !TileOffsets_global || !bitmap)
+        return -4;
+    if (M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
+        return -2;
+    int* sizes = static_cast<int*>(read_exact(OutputSizesFileName, sizeof(int), 4));
+    if (sizes == nullptr)
+        return -1;
+    const long G = (long)(M / 64) * (K / 64);
+    const int  count = sizes[0];
+    const bool fits  = count >= 0 && count % 8 == 0 && sizes[1] == G + 1 && sizes[2] == 4 * G && sizes[3] == 64 * G;
+    std::free(sizes);
+    if (!fits)
+        return -2;
+    uint16_t* vals   = static_cast<uint16_t*>(read_exact(Compressed_ValFileName, sizeof(uint16_t), (size_t)count));
+    int*      global = static_cast<int*>(read_exact(TileOffsets_globalFileName, sizeof(int), (size_t)G + 1));
+    int*      median = static_cast<int*>(read_exact(TileOffsets_medianFileName, sizeof(int), 4 * (size_t)G));
+    uint64_t* bm     = static_cast<uint64_t*>(read_exact(bitmapFileName, sizeof(uint64_t), 64 * (size_t)G));
+    int*      nnz    = static_cast<int*>(read_exact(max_nnz_intileFileName, sizeof(int), 1));
+    int       rc     = (int)G;
+    if (!vals || !global || !median || !bm || !nnz)
+        rc = -1;
+    else if (global[0] != 0 || global[G] != count)
+        rc = -2; // the offsets do not describe the values file
+    else
+        for (long g = 0; g < G && rc >= 0; ++g)
+            if (global[g + 1] < global[g] || (global[g + 1] - global[g]) % 8 != 0 || global[g + 1] - global[g] > 4096)
+                rc = -2;
+    if (rc < 0) {
+        std::free(vals), std::free(global), std::free(median), std::free(bm), std::free(nnz);
+        return rc;
+    }
+    *Compressed_Val     = vals;
+    *TileOffsets_global = global;
+    *bitmap             = bm;
+    if (TileOffsets_median != nullptr)
+        *TileOffsets_median = median;
+    else
+        std::free(median);
+    if (max_nnz_intile != nullptr)
+        *max_nnz_intile = *nnz;
+    std::free(nnz);
+    if (val_count != nullptr)
+        *val_count = count;
+    return rc;
+}

@@ -3,12 +3,15 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
+#include <dlfcn.h>
+
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <map>
 #include <memory>
 #include <mutex>
+#include <string>
 #include <tuple>
 #include <vector>
 
@@ -105,17 +108,18 @@ int auto_split_k(int M, int N, int K)
 
 // Measured choices that take precedence over the cost model (the role of the reference's SplitKDict,
 // end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:23, and of the SPLIT_K array of
-// kernel_benchmark/run_all_main.sh:5): a table keyed by (M, N, K), filled by SpMM_SplitK_TableSet or from a text
-// file of "M N K Split_K" lines.  SPMM_SPLITK_TABLE in the environment names a file that is loaded on first use.
-// Readers never lock: the table is an immutable snapshot behind an atomic pointer; a writer (rare: table set-up)
-// copies it under the mutex, changes the copy and publishes it.  Superseded snapshots stay alive until the process
-// ends, so a reader that still holds one is safe.
+// kernel_benchmark/run_all_main.sh:5): a table keyed by (M, N, K), filled by SpMM_SplitK_TableSet/SetMany or from a
+// text file of "M N K Split_K" lines.  On first use a file is loaded: the one SPMM_SPLITK_TABLE names, or, when the
+// variable is not set, the measured table shipped beside the library (../tuned/splitk_mi355x.txt from the
+// library's own directory); SPMM_SPLITK_TABLE set to an empty string loads nothing.
+// The table is an immutable snapshot behind a shared pointer: a reader takes a reference for the length of its
+// look-up, a writer (rare: table set-up) copies the snapshot under the mutex, changes the copy and publishes it;
+// a superseded snapshot is freed when its last reader lets go, so a process that retunes does not grow.
 using SplitMap = std::map<std::tuple<int, int, int>, int>;
 struct SplitTable {
-    std::mutex                               lock;     // writers only
-    std::atomic<const SplitMap*>             current{nullptr};
-    std::vector<std::unique_ptr<SplitMap>>   versions; // every snapshot ever published (guarded by lock)
-    std::atomic<bool>                        env_checked{false};
+    std::mutex                      lock;    // writers only
+    std::shared_ptr<const SplitMap> current; // read and written with std::atomic_load / std::atomic_store
+    std::atomic<bool>               env_checked{false};
 };
 SplitTable& split_table()
 {
@@ -127,11 +131,10 @@ SplitTable& split_table()
 template <typename F>
 void publish_locked(SplitTable& t, F change)
 {
-    const SplitMap* cur = t.current.load(std::memory_order_acquire);
-    auto            nxt = std::make_unique<SplitMap>(cur ? *cur : SplitMap());
+    std::shared_ptr<const SplitMap> cur = std::atomic_load_explicit(&t.current, std::memory_order_acquire);
+    auto                            nxt = std::make_shared<SplitMap>(cur ? *cur : SplitMap());
     change(*nxt);
-    t.current.store(nxt.get(), std::memory_order_release);
-    t.versions.push_back(std::move(nxt));
+    std::atomic_store_explicit(&t.current, std::shared_ptr<const SplitMap>(std::move(nxt)), std::memory_order_release);
 }
 
 // returns the number of entries read, or -1 when the file cannot be opened, -2 on a malformed line (nothing is
@@ -164,6 +167,18 @@ int load_split_table_locked(SplitTable& t, const char* path)
     return (int)read.size();
 }
 
+// Path of the table shipped with the library: <directory of libSpMM_API.so>/../tuned/splitk_mi355x.txt.
+std::string shipped_table_path()
+{
+    Dl_info info;
+    if (!dladdr(reinterpret_cast<const void*>(&split_table), &info) || info.dli_fname == nullptr)
+        return std::string();
+    std::string       lib(info.dli_fname);
+    const std::size_t slash = lib.find_last_of('/');
+    const std::string dir   = slash == std::string::npos ? std::string(".") : lib.substr(0, slash);
+    return dir + "/../tuned/splitk_mi355x.txt";
+}
+
 void check_env_table_once(SplitTable& t)
 {
     if (t.env_checked.load(std::memory_order_acquire))
@@ -172,12 +187,18 @@ void check_env_table_once(SplitTable& t)
     if (t.env_checked.load(std::memory_order_relaxed))
         return;
     if (const char* e = std::getenv("SPMM_SPLITK_TABLE")) {
-        const int n = load_split_table_locked(t, e);
-        if (n < 0) {
-            std::printf("MM_Sparse_API Warning: SPMM_SPLITK_TABLE=%s %s; using the built-in choice.\n", e,
-                        n == -1 ? "cannot be opened" : "has a malformed line");
-            std::fflush(stdout);
+        if (*e != 0) {
+            const int n = load_split_table_locked(t, e);
+            if (n < 0) {
+                std::printf("MM_Sparse_API Warning: SPMM_SPLITK_TABLE=%s %s; using the built-in choice.\n", e,
+                            n == -1 ? "cannot be opened" : "has a malformed line");
+                std::fflush(stdout);
+            }
         }
+    } else {
+        const std::string shipped = shipped_table_path();
+        if (!shipped.empty())
+            (void)load_split_table_locked(t, shipped.c_str()); // absent or unreadable: the cost model stands
     }
     t.env_checked.store(true, std::memory_order_release);
 }
@@ -186,7 +207,7 @@ int split_k_for(int M, int N, int K)
 {
     SplitTable& t = split_table();
     check_env_table_once(t);
-    if (const SplitMap* m = t.current.load(std::memory_order_acquire)) {
+    if (std::shared_ptr<const SplitMap> m = std::atomic_load_explicit(&t.current, std::memory_order_acquire)) {
         auto it = m->find(std::make_tuple(M, N, K));
         if (it != m->end())
             return clamp_split_k(it->second, K);
@@ -264,13 +285,40 @@ extern "C" int SpMM_SplitK_Auto(int M, int N, int K)
     return split_k_for(M, N, K);
 }
 
+extern "C" int SpMM_SplitK_CostModel(int M, int N, int K)
+{
+    if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
+        return 1;
+    return clamp_split_k(auto_split_k(M, N, K), K);
+}
+
 extern "C" int SpMM_SplitK_TableSet(int M, int N, int K, int Split_K)
 {
     if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0 || Split_K < 1)
         return (int)hipErrorInvalidValue;
-    SplitTable&                 t = split_table();
+    SplitTable& t = split_table();
+    check_env_table_once(t); // the start-up file first: it must not undo this entry later
     std::lock_guard<std::mutex> g(t.lock);
     publish_locked(t, [&](SplitMap& m) { m[std::make_tuple(M, N, K)] = Split_K; });
+    return 0;
+}
+
+extern "C" int SpMM_SplitK_TableSetMany(const int* entries, int count)
+{
+    if (count < 0 || (count > 0 && entries == nullptr))
+        return (int)hipErrorInvalidValue;
+    for (int i = 0; i < count; ++i) {
+        const int M = entries[4 * i], N = entries[4 * i + 1], K = entries[4 * i + 2], sk = entries[4 * i + 3];
+        if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0 || sk < 1)
+            return (int)hipErrorInvalidValue; // nothing is recorded
+    }
+    SplitTable& t = split_table();
+    check_env_table_once(t);
+    std::lock_guard<std::mutex> g(t.lock);
+    publish_locked(t, [&](SplitMap& m) {
+        for (int i = 0; i < count; ++i)
+            m[std::make_tuple(entries[4 * i], entries[4 * i + 1], entries[4 * i + 2])] = entries[4 * i + 3];
+    });
     return 0;
 }
 
@@ -278,7 +326,8 @@ extern "C" int SpMM_SplitK_TableLoad(const char* path)
 {
     if (path == nullptr)
         return -1;
-    SplitTable&                 t = split_table();
+    SplitTable& t = split_table();
+    check_env_table_once(t);
     std::lock_guard<std::mutex> g(t.lock);
     return load_split_table_locked(t, path);
 }
@@ -287,8 +336,9 @@ extern "C" int SpMM_SplitK_TableSave(const char* path)
 {
     if (path == nullptr)
         return -1;
-    const SplitMap* m = split_table().current.load(std::memory_order_acquire);
-    std::FILE*      f = std::fopen(path, "w");
+    check_env_table_once(split_table());
+    std::shared_ptr<const SplitMap> m = std::atomic_load_explicit(&split_table().current, std::memory_order_acquire);
+    std::FILE*                      f = std::fopen(path, "w");
     if (!f)
         return -1;
     std::fprintf(f, "# M N K Split_K\n");
@@ -304,7 +354,8 @@ extern "C" int SpMM_SplitK_TableSave(const char* path)
 
 extern "C" void SpMM_SplitK_TableClear(void)
 {
-    SplitTable&                 t = split_table();
+    SplitTable& t = split_table();
+    check_env_table_once(t);
     std::lock_guard<std::mutex> g(t.lock);
     publish_locked(t, [](SplitMap& m) { m.clear(); });
 }
@@ -432,8 +483,15 @@ extern "C" int SpMM_SplitK_API_NoAlloc(hipStream_t stream, const void* values, c
 {
     if (int e = check_shape(M, N, K))
         return refuse(e);
-    const int    sk   = Split_K <= 0 ? split_k_for(M, N, K) : clamp_split_k(Split_K, K);
-    const size_t need = sk > 1 ? sizeof(float) * (size_t)M * (size_t)N * (size_t)sk : 0;
+    int          sk   = Split_K <= 0 ? split_k_for(M, N, K) : clamp_split_k(Split_K, K);
+    const size_t slab = sizeof(float) * (size_t)M * (size_t)N;
+    if (Split_K <= 0 && sk > 1 && slab * (size_t)sk > (size_t)SPMM_NOALLOC_SCRATCH_BYTES) {
+        // the library's own choice gives way to the largest split whose partial sums fit; an unsplit K needs none
+        sk = (int)((size_t)SPMM_NOALLOC_SCRATCH_BYTES / slab);
+        if (sk < 2)
+            sk = 1;
+    }
+    const size_t need = sk > 1 ? slab * (size_t)sk : 0;
     if (need > (size_t)SPMM_NOALLOC_SCRATCH_BYTES) {
         std::printf("MM_Sparse_API Error: M=%d N=%d Split_K=%d needs %zu bytes of partial sums; "
                     "SpMM_SplitK_API_NoAlloc holds at most %zu!\n",
@@ -453,6 +511,79 @@ extern "C" int SpMM_SplitK_API_NoAlloc(hipStream_t stream, const void* values, c
         }
     }
     return run(stream, values, bitmaps, offsets, X, C, M, N, K, ws, sk, /*fp32_partials=*/true);
+}
+
+extern "C" int SpMM_SplitK_AutoNoAlloc(int M, int N, int K)
+{
+    if (!supported_n(N) || M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
+        return 1;
+    int          sk   = split_k_for(M, N, K);
+    const size_t slab = sizeof(float) * (size_t)M * (size_t)N;
+    if (sk > 1 && slab * (size_t)sk > (size_t)SPMM_NOALLOC_SCRATCH_BYTES) {
+        sk = (int)((size_t)SPMM_NOALLOC_SCRATCH_BYTES / slab);
+        if (sk < 2)
+            sk = 1;
+    }
+    return sk;
+}
+
+// ---- the six weight files -> device arrays (the consumer side of Our_GenSparseMatrixBinFile) -------------------
+extern "C" void SpMM_FreeWeights(void* values_d, int* offsets_d, int* median_d, uint64_t* bitmaps_d, int* max_nnz_d)
+{
+    void* all[5] = {values_d, offsets_d, median_d, bitmaps_d, max_nnz_d};
+    for (void* p : all)
+        if (p != nullptr)
+            (void)hipFree(p);
+}
+
+extern "C" int SpMM_LoadWeightFiles(const char* Compressed_ValFileName, const char* TileOffsets_globalFileName,
+                                    const char* TileOffsets_medianFileName, const char* bitmapFileName,
+                                    const char* max_nnz_intileFileName, const char* OutputSizesFileName, int M, int K,
+                                    void** values_d, int** offsets_d, int** median_d, uint64_t** bitmaps_d,
+                                    int** max_nnz_d, int* val_count)
+{
+    if (values_d == nullptr || offsets_d == nullptr || bitmaps_d == nullptr)
+        return -4;
+    uint16_t* vals   = nullptr;
+    int *     global = nullptr, *median = nullptr;
+    uint64_t* bitmap = nullptr;
+    int       max_nnz = 0, count = 0;
+    const int G = SpMM_ReadWeightFiles(Compressed_ValFileName, TileOffsets_globalFileName, TileOffsets_medianFileName,
+                                       bitmapFileName, max_nnz_intileFileName, OutputSizesFileName, M, K, &vals,
+                                       &global, &median, &bitmap, &max_nnz, &count);
+    if (G < 0)
+        return G;
+    void *    dv = nullptr, *dg = nullptr, *dm = nullptr, *db = nullptr, *dn = nullptr;
+    const size_t bytes_v = sizeof(uint16_t) * (size_t)count, bytes_g = sizeof(int) * ((size_t)G + 1),
+                 bytes_m = sizeof(int) * 4 * (size_t)G, bytes_b = sizeof(uint64_t) * 64 * (size_t)G;
+    hipError_t err = hipMalloc(&dv, bytes_v ? bytes_v : 16); // an all-zero matrix still gets a valid pointer
+    if (err == hipSuccess) err = hipMalloc(&dg, bytes_g);
+    if (err == hipSuccess) err = hipMalloc(&db, bytes_b);
+    if (err == hipSuccess && median_d != nullptr) err = hipMalloc(&dm, bytes_m);
+    if (err == hipSuccess && max_nnz_d != nullptr) err = hipMalloc(&dn, sizeof(int));
+    if (err == hipSuccess && bytes_v) err = hipMemcpy(dv, vals, bytes_v, hipMemcpyHostToDevice);
+    if (err == hipSuccess) err = hipMemcpy(dg, global, bytes_g, hipMemcpyHostToDevice);
+    if (err == hipSuccess) err = hipMemcpy(db, bitmap, bytes_b, hipMemcpyHostToDevice);
+    if (err == hipSuccess && dm != nullptr) err = hipMemcpy(dm, median, bytes_m, hipMemcpyHostToDevice);
+    if (err == hipSuccess && dn != nullptr) err = hipMemcpy(dn, &max_nnz, sizeof(int), hipMemcpyHostToDevice);
+    std::free(vals), std::free(global), std::free(median), std::free(bitmap);
+    if (err != hipSuccess) {
+        std::printf("MM_Sparse_API Error: SpMM_LoadWeightFiles: %s!\n", hipGetErrorString(err));
+        std::fflush(stdout);
+        SpMM_FreeWeights(dv, static_cast<int*>(dg), static_cast<int*>(dm), static_cast<uint64_t*>(db),
+                         static_cast<int*>(dn));
+        return -5;
+    }
+    *values_d  = dv;
+    *offsets_d = static_cast<int*>(dg);
+    *bitmaps_d = static_cast<uint64_t*>(db);
+    if (median_d != nullptr)
+        *median_d = static_cast<int*>(dm);
+    if (max_nnz_d != nullptr)
+        *max_nnz_d = static_cast<int*>(dn);
+    if (val_count != nullptr)
+        *val_count = count;
+    return G;
 }
 
 extern "C" void SpMM_TimeNextCall(hipEvent_t before_main, hipEvent_t after_main)

@@ -25,19 +25,35 @@ __all__ = ["sparse_linear", "SparseLinearModule"]
 
 @torch.library.custom_op("spmspm_amd::sparse_linear", mutates_args=(), device_types="cuda")
 def sparse_linear(x: torch.Tensor, values: torch.Tensor, bitmaps: torch.Tensor, offsets: torch.Tensor,
-                  bias: Optional[torch.Tensor], M: int, split_k: int, activation: int) -> torch.Tensor:
+                  bias: Optional[torch.Tensor], M: int, split_k: int, activation: int,
+                  nnz: int = -1) -> torch.Tensor:
     """y[N][M] = act(W x + bias) for the compressed W given by (values, bitmaps, offsets).
 
     x [N][K] fp16 contiguous; values int16/fp16 (compact non-zeros), bitmaps int64 (64 per group tile), offsets
-    int32 (G+1); bias fp16 [M] or None; split_k <= 0 lets the library choose; activation 0 none, 1 ReLU, 2 GELU."""
-    if x.dim() != 2 or x.dtype != torch.float16 or not x.is_contiguous():
-        raise ValueError("x must be a contiguous [N][K] fp16 tensor")
+    int32 (G+1); bias fp16 [M] or None; split_k <= 0 lets the library choose; activation 0 none, 1 ReLU, 2 GELU;
+    nnz, when not negative, is offsets[G] as the caller knows it (the number of halves `values` must hold), checked
+    here without reading device memory.  Every check happens on the host before anything is launched: the kernels
+    trust their pointers."""
+    if x.dim() != 2 or x.dtype != torch.float16 or not x.is_contiguous() or not x.is_cuda:
+        raise ValueError("x must be a contiguous [N][K] fp16 tensor on the GPU")
     N, K = x.shape
     G = offsets.numel() - 1
     if M <= 0 or M % 64 or K % 64 or G != (M // 64) * (K // 64) or bitmaps.numel() != 64 * G:
         raise ValueError(f"compressed arrays do not describe a {M}x{K} matrix")
+    if offsets.dtype != torch.int32 or bitmaps.dtype != torch.int64 or values.dtype not in (torch.int16, torch.float16):
+        raise ValueError("offsets must be int32, bitmaps int64 and values int16 or fp16 "
+                         f"(got {offsets.dtype}, {bitmaps.dtype}, {values.dtype})")
+    for name, t in (("values", values), ("bitmaps", bitmaps), ("offsets", offsets), ("bias", bias)):
+        if t is None:
+            continue
+        if t.device != x.device:
+            raise ValueError(f"{name} is on {t.device}, x on {x.device}: all operands must share x's device")
+        if not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous")
+    if nnz >= 0 and values.numel() < nnz:
+        raise ValueError(f"values holds {values.numel()} halves, the offsets end at {nnz}")
     fused = bias is not None or activation != A.ACT_NONE
-    if bias is not None and (bias.numel() != M or bias.dtype != torch.float16 or not bias.is_contiguous()):
+    if bias is not None and (bias.numel() != M or bias.dtype != torch.float16):
         raise ValueError("bias must be M contiguous fp16 values")
     sk = split_k if split_k > 0 else A.SpMM_SplitK_Auto(M, N, K)  # resolved once: the workspace matches the call
     need = (A.SpMM_WorkspaceBytesBiasAct if fused else A.SpMM_WorkspaceBytes)(M, N, K, sk)
@@ -57,7 +73,7 @@ def sparse_linear(x: torch.Tensor, values: torch.Tensor, bitmaps: torch.Tensor, 
 
 
 @sparse_linear.register_fake
-def _(x, values, bitmaps, offsets, bias, M, split_k, activation):
+def _(x, values, bitmaps, offsets, bias, M, split_k, activation, nnz=-1):
     return x.new_empty((x.shape[0], M))
 
 
@@ -68,6 +84,10 @@ class SparseLinearModule(torch.nn.Module):
     def __init__(self, M, K, values, bitmaps, offsets, bias=None, activation=A.ACT_NONE, split_k=0):
         super().__init__()
         self.M, self.K, self.activation, self.split_k = int(M), int(K), int(activation), int(split_k)
+        # offsets[G], read once here: the operator then checks `values` against it without touching device memory
+        self.nnz = int(offsets[-1].item()) if offsets.numel() else 0
+        if values.numel() < self.nnz:
+            raise ValueError(f"values holds {values.numel()} halves, the offsets end at {self.nnz}")
         self.register_buffer("values", values)
         self.register_buffer("bitmaps", bitmaps)
         self.register_buffer("offsets", offsets)
@@ -93,7 +113,7 @@ class SparseLinearModule(torch.nn.Module):
 
     def forward(self, x):
         return torch.ops.spmspm_amd.sparse_linear(x, self.values, self.bitmaps, self.offsets, self.bias, self.M,
-                                                  self.split_k, self.activation)
+                                                  self.split_k, self.activation, self.nnz)
 
     def extra_repr(self):
         return f"M={self.M}, K={self.K}, split_k={self.split_k}, activation={self.activation}"

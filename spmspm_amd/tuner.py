@@ -77,21 +77,8 @@ def tune_shape(M, N, K, sparsity=0.6, candidates=None, device="cuda:0", iters=30
 
 
 def _cost_model_choice(M, N, K):
-    """What the built-in cost model picks for a shape, with the table left exactly as it was: the table is saved
-    to a temporary file, emptied for the question and loaded back (entries of the user, of SPMM_SPLITK_TABLE and of
-    earlier shapes alike)."""
-    import os
-    import tempfile
-    fd, path = tempfile.mkstemp(suffix=".splitk")
-    os.close(fd)
-    try:
-        A.SpMM_SplitK_TableSave(path)
-        A.SpMM_SplitK_TableClear()
-        model = A.SpMM_SplitK_Auto(M, N, K)
-        A.SpMM_SplitK_TableLoad(path)
-    finally:
-        os.unlink(path)
-    return model
+    """What the built-in cost model picks for a shape (the table is not consulted)."""
+    return A.SpMM_SplitK_CostModel(M, N, K)
 
 
 def tune(shapes, N, sparsity=0.6, record=True, log=None, **kw):

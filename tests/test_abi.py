@@ -22,7 +22,9 @@ def test_header_declares_the_expected_entry_points():
               "Our_GenSparseMatrixBinFile", "SpMM_SplitK_Auto", "SpMM_WorkspaceBytes", "SpMM_Version", "SpMM_TimeNextCall",
               "SpMM_SplitK_API_BiasAct", "SpMM_WorkspaceBytesBiasAct", "SpMM_EncodeDevice_Bitmaps",
               "SpMM_EncodeDevice_Values", "SpMM_SplitK_TableSet", "SpMM_SplitK_TableLoad", "SpMM_SplitK_TableSave",
-              "SpMM_SplitK_TableClear", "SpMM_SplitK_API_NoAlloc", "SpMM_SplitK_API_Sized", "SpMM_KernelName"):
+              "SpMM_SplitK_TableClear", "SpMM_SplitK_API_NoAlloc", "SpMM_SplitK_API_Sized", "SpMM_KernelName",
+              "SpMM_SplitK_TableSetMany", "SpMM_SplitK_CostModel", "SpMM_SplitK_AutoNoAlloc", "SpMM_ReadWeightFiles",
+              "SpMM_LoadWeightFiles", "SpMM_FreeWeights"):
         assert n in names
 
 
@@ -101,8 +103,9 @@ def test_split_table_overrides_the_cost_model_and_round_trips_through_a_file(tmp
 def test_shipped_split_table_loads_and_covers_the_decode_widths():
     """The measured table in spmspm_amd/tuned/ parses, lists the OPT-13B, OPT-30B and OPT-66B linears at N = 8, 16,
     32, 64 and 128, and takes precedence over the cost model once loaded."""
-    path = os.path.join(ROOT, "spmspm_amd", "tuned", "splitk_mi355x_s60.txt")
+    path = os.path.join(ROOT, "spmspm_amd", "tuned", "splitk_mi355x.txt")
     try:
+        S.SpMM_SplitK_TableClear()
         assert S.SpMM_SplitK_TableLoad(path) == 60
         for M, K in [(15360, 5120), (5120, 5120), (20480, 5120), (5120, 20480), (28672, 7168), (7168, 7168),
                      (21504, 7168), (7168, 28672), (27648, 9216), (9216, 9216), (36864, 9216), (9216, 36864)]:
@@ -134,6 +137,75 @@ def test_split_table_file_named_in_the_environment_is_loaded_on_first_use(tmp_pa
     env["SPMM_SPLITK_TABLE"] = str(tmp_path / "missing.txt")
     r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True)
     assert "cannot be opened" in r.stdout and int(r.stdout.split()[-2]) >= 1
+
+
+def test_shipped_table_is_loaded_by_default_and_an_empty_variable_switches_it_off():
+    """Without SPMM_SPLITK_TABLE the library finds tuned/splitk_mi355x.txt beside its own directory on first use; with
+    the variable set to an empty string the cost model stands alone."""
+    import subprocess
+    import sys
+    path = os.path.join(ROOT, "spmspm_amd", "tuned", "splitk_mi355x.txt")
+    table = {}
+    for line in open(path):
+        if line.strip() and not line.startswith("#"):
+            m, n, k, sk = map(int, line.split())
+            table[(m, n, k)] = sk
+    code = ("import spmspm_amd as S\n"
+            "for m, n, k in %r:\n"
+            "    print(m, n, k, S.SpMM_SplitK_Auto(m, n, k), S.SpMM_SplitK_CostModel(m, n, k))" % (sorted(table),))
+    env = {k: v for k, v in os.environ.items() if k != "SPMM_SPLITK_TABLE"}
+    env["PYTHONPATH"] = ROOT
+    rows = [tuple(map(int, l.split())) for l in
+            subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True).stdout.splitlines()]
+    assert len(rows) == len(table)
+    assert all(auto == table[(m, n, k)] for m, n, k, auto, _ in rows)
+    assert any(auto != model for _, _, _, auto, model in rows)  # the table does overrule the model somewhere
+    env["SPMM_SPLITK_TABLE"] = ""
+    rows = [tuple(map(int, l.split())) for l in
+            subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True).stdout.splitlines()]
+    assert all(auto == model for _, _, _, auto, model in rows)
+
+
+def test_table_set_many_records_all_or_nothing():
+    import pytest
+    S.SpMM_SplitK_TableClear()
+    try:
+        S.SpMM_SplitK_TableSetMany([(4096, 16, 4096, 3), (8192, 32, 4096, 5)])
+        assert S.SpMM_SplitK_Auto(4096, 16, 4096) == 3 and S.SpMM_SplitK_Auto(8192, 32, 4096) == 5
+        with pytest.raises(ValueError):
+            S.SpMM_SplitK_TableSetMany([(4096, 8, 4096, 7), (100, 16, 64, 2)])  # second entry is no shape the library runs
+        assert S.SpMM_SplitK_Auto(4096, 8, 4096) == S.SpMM_SplitK_CostModel(4096, 8, 4096)
+        S.SpMM_SplitK_TableSetMany([])
+        # many updates in a row leave one table, not one copy per update alive
+        for i in range(2000):
+            S.SpMM_SplitK_TableSet(4096, 16, 4096, 1 + i % 7)
+        assert S.SpMM_SplitK_Auto(4096, 16, 4096) == 1 + 1999 % 7
+    finally:
+        S.SpMM_SplitK_TableClear()
+
+
+def test_no_alloc_entry_point_clamps_its_own_split_and_refuses_an_explicit_one(capfd):
+    """With Split_K <= 0 the library's choice gives way to the largest split whose fp32 partial sums fit the 32 MiB
+    array; an explicit Split_K beyond it is refused before anything touches the device."""
+    M, N, K = 20480, 128, 5120
+    S.SpMM_SplitK_TableClear()
+    try:
+        S.SpMM_SplitK_TableSet(M, N, K, 6)  # 4*M*N*6 = 60 MiB of partial sums
+        assert S.SpMM_SplitK_Auto(M, N, K) == 6
+        fit = S.SpMM_SplitK_AutoNoAlloc(M, N, K)
+        assert fit == 3 and 4 * M * N * fit <= S.NOALLOC_SCRATCH_BYTES < 4 * M * N * (fit + 1)
+        capfd.readouterr()
+        rc = S.library().SpMM_SplitK_API_NoAlloc(None, None, None, None, None, None, M, N, K, 0)
+        out = capfd.readouterr().out
+        assert "holds at most" not in out  # not refused for its size; without a GPU the device look-up fails instead
+        assert rc != 1 or "scratch array" in out
+        assert S.library().SpMM_SplitK_API_NoAlloc(None, None, None, None, None, None, M, N, K, 6) == 1
+        assert "holds at most" in capfd.readouterr().out
+        # a single slab beyond the array: the automatic call runs unsplit
+        assert S.SpMM_SplitK_AutoNoAlloc(36864, 256, 9216) == 1
+        assert S.SpMM_SplitK_AutoNoAlloc(5120, 16, 5120) == S.SpMM_SplitK_Auto(5120, 16, 5120)
+    finally:
+        S.SpMM_SplitK_TableClear()
 
 
 def test_tuner_candidates_and_presets():
@@ -180,6 +252,8 @@ def test_kernel_name_follows_the_dispatch():
     assert name(128, 64, 4096, 2) == "spmm::spmm_bitmap_rows<4, true>"   # fewer than 256 rows
     assert name(9216, 256, 36864, 7) == "spmm::spmm_bitmap_wide<8, true>"
     assert name(9216, 24, 36864, 1) == "" and name(100, 16, 64, 1) == ""
+    # the name is that of SpMM_SplitK_API / _Sized / _NoAlloc: fp32 partial sums exactly when K is split
+    assert name(5120, 16, 5120, 1).endswith("false>") and name(5120, 16, 5120, 2).endswith("true>")
 
 
 def test_row_count_limit_is_reported(capfd):

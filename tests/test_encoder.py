@@ -103,6 +103,49 @@ def test_weight_files_byte_layout(tmp_path, oracle):
     back = S.load_weight_files(*names, M, K)
     assert np.array_equal(back.values, e["values"]) and np.array_equal(back.bitmaps, e["bitmap"][:64 * G])
     assert np.array_equal(back.tile_counts, e["tile_cnt"][:64 * G])
+    # the library's own reader (C ABI) returns the same arrays
+    read = S.SpMM_ReadWeightFiles(*names, M, K)
+    assert read.num_gtiles == G and read.max_nnz == oracle.round_max_nnz(e["max_nnz"])
+    assert np.array_equal(read.values, e["values"]) and np.array_equal(read.bitmaps, e["bitmap"][:64 * G])
+    assert np.array_equal(read.offsets, e["global"]) and np.array_equal(read.median, e["median"])
+    assert np.array_equal(read.tile_counts, e["tile_cnt"][:64 * G])
+
+
+def test_weight_file_reader_reports_what_is_wrong(tmp_path, oracle):
+    """SpMM_ReadWeightFiles never ends the process: a missing or truncated file is -1 (OSError here), files that do
+    not match M and K or each other are -2 (ValueError)."""
+    from spmspm_amd.synthetic import make_weight
+    M, K = 128, 192
+    W = make_weight(M, K, 0.5, seed=3)
+    dense = tmp_path / "w.bin"
+    W.tofile(dense)
+    names = [str(tmp_path / f"w.{s}.bin") for s in ("NZWeights", "gtile", "mtile", "ltile", "intile", "OutputSizes")]
+    S.Our_GenSparseMatrixBinFile(str(dense), M, K, *names)
+    assert S.SpMM_ReadWeightFiles(*names, M, K).num_gtiles == 6
+    with pytest.raises(ValueError):
+        S.SpMM_ReadWeightFiles(*names, M, K + 64)          # sizes file written for another shape
+    with pytest.raises(ValueError):
+        S.SpMM_ReadWeightFiles(*names, M + 1, K)           # not a multiple of 64
+    vals = np.fromfile(names[0], np.uint16)
+    vals[:-8].tofile(names[0])                             # values file eight halves short
+    with pytest.raises(OSError):
+        S.SpMM_ReadWeightFiles(*names, M, K)
+    vals.tofile(names[0])
+    off = np.fromfile(names[1], np.int32)
+    bad = off.copy()
+    bad[2] += 4                                            # a run that is no multiple of eight
+    bad.tofile(names[1])
+    with pytest.raises(ValueError):
+        S.SpMM_ReadWeightFiles(*names, M, K)
+    off.tofile(names[1])
+    os.unlink(names[3])
+    with pytest.raises(OSError):
+        S.SpMM_ReadWeightFiles(*names, M, K)
+    # an all-zero matrix: an empty values file is a valid one
+    np.zeros((64, 64), np.float16).tofile(dense)
+    S.Our_GenSparseMatrixBinFile(str(dense), 64, 64, *names)
+    z = S.SpMM_ReadWeightFiles(*names, 64, 64)
+    assert z.values.size == 0 and list(z.offsets) == [0, 0]
 
 
 def test_weight_file_missing_input_exits_like_reference(tmp_path):

@@ -1,4 +1,5 @@
-"""Device encoder (SpMM_EncodeDevice_*) against the host encoder, bit for bit, and its output fed to the SpMM."""
+"""Device encoder (SpMM_EncodeDevice_*) against the CPU oracle (the restatement of csrc/SpMM_API.cuh:112-241), the
+committed golden encodings and the host encoder, bit for bit, and its output fed to the SpMM."""
 import numpy as np
 import pytest
 
@@ -33,18 +34,41 @@ def _special_matrix(M, K, seed):
 
 @pytest.mark.parametrize("M,K,sparsity", [(64, 64, 0.5), (128, 192, 0.7), (512, 1024, 0.9), (1024, 256, 0.0),
                                           (256, 256, 1.0), (2048, 4096, 0.6), (65536, 64, 0.5)])
-def test_device_encoder_is_bit_identical_to_the_host_encoder(torch, M, K, sparsity):
+def test_device_encoder_is_bit_identical_to_the_oracle_and_the_host_encoder(torch, oracle, M, K, sparsity):
     W = _special_matrix(M, K, seed=M + K) if (M >= 192 and K >= 128) else make_weight(M, K, sparsity, seed=M + K)
     if sparsity == 1.0:
         W[:] = 0
+    want = oracle.encode(W, M, K)
     comp = S.InitSparseMatrixA_bitmap(W)
     Wd = torch.from_numpy(W.view(np.int16).copy()).to("cuda:0").view(torch.float16)
     print(f"case M={M} K={K} s={sparsity}", flush=True)
     values, bitmaps, offsets = S.InitSparseMatrixA_bitmap_device(Wd)
     torch.cuda.synchronize()
-    assert np.array_equal(offsets.cpu().numpy(), comp.offsets)
-    assert np.array_equal(bitmaps.cpu().numpy().view(np.uint64), comp.bitmaps)
-    assert np.array_equal(values.cpu().numpy().view(np.uint16), comp.values)
+    got_o, got_b, got_v = offsets.cpu().numpy(), bitmaps.cpu().numpy().view(np.uint64), values.cpu().numpy().view(np.uint16)
+    assert np.array_equal(got_o, want["global"])
+    assert np.array_equal(got_b, want["bitmap"])
+    assert np.array_equal(got_v, want["values"])
+    assert np.array_equal(got_o, comp.offsets) and np.array_equal(got_b, comp.bitmaps) and np.array_equal(got_v, comp.values)
+
+
+def test_device_encoder_reproduces_the_golden_encodings(torch, golden):
+    """Every committed golden input whose shape the device encoder takes (multiples of 64): W -> device -> arrays must
+    be the arrays the reference's own encoder wrote into the fixture."""
+    ran = 0
+    for name, case in golden.items():
+        W = case["W"]
+        M, K = W.shape
+        if M % 64 or K % 64:
+            continue
+        print(f"golden {name} {M}x{K}", flush=True)
+        Wd = torch.from_numpy(W.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+        values, bitmaps, offsets = S.InitSparseMatrixA_bitmap_device(Wd)
+        torch.cuda.synchronize()
+        assert np.array_equal(offsets.cpu().numpy(), case["offsets"]), name
+        assert np.array_equal(bitmaps.cpu().numpy().view(np.uint64), case["bitmaps"]), name
+        assert np.array_equal(values.cpu().numpy().view(np.uint16), case["values"]), name
+        ran += 1
+    assert ran >= 7
 
 
 def test_device_encoded_weights_multiply_correctly(torch, oracle):
@@ -70,11 +94,13 @@ def test_device_encoder_rejects_ragged_shapes(torch, capfd):
     assert L.SpMM_EncodeDevice_Values(None, t.data_ptr(), 64, 70, t.data_ptr(), t.data_ptr()) == S.api.HIP_ERROR_INVALID_VALUE
 
 
-def test_device_encoder_offsets_scan_across_many_blocks(torch):
+def test_device_encoder_offsets_scan_across_many_blocks(torch, oracle):
     """More than 1024 group tiles, not a multiple of 1024: the in-place running sum crosses block boundaries."""
     M, K = 64 * 37, 64 * 61  # 2257 group tiles
     W = make_weight(M, K, 0.8, seed=9)
     comp = S.InitSparseMatrixA_bitmap(W)
+    want = oracle.encode(W, M, K)
+    assert np.array_equal(comp.offsets, want["global"]) and np.array_equal(comp.values, want["values"])
     Wd = torch.from_numpy(W.view(np.int16).copy()).to("cuda:0").view(torch.float16)
     values, bitmaps, offsets = S.InitSparseMatrixA_bitmap_device(Wd)
     torch.cuda.synchronize()

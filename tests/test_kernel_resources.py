@@ -25,12 +25,3 @@ def test_main_kernel_occupancy_budget():
             assert r["vgpr"] <= limit[key], (name, r)
             seen += 1
     assert seen == 6
-
-
-def test_ablation_patches_still_apply(tmp_path):
-    """`python -m spmspm_amd.ablate` switches parts of the main kernel off by patching a copy of its source; every
-    patch must still find its place after the kernel has changed (the copy is made and patched here, not compiled)."""
-    from spmspm_amd import ablate
-    ablate.patched_sources(str(tmp_path))
-    text = (tmp_path / "spmm_kernels.hiph").read_text()
-    assert "ABL_NOX" in text and "ABL_NODECODE" in text

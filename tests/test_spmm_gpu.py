@@ -488,7 +488,7 @@ OPT13B_LINEARS = [("opt13b_qkv", 15360, 5120), ("opt13b_out", 5120, 5120), ("opt
 
 def _tuned_split(M, N, K):
     """Split_K of the shipped measured table (spmspm_amd/tuned/), or None if the shape is not listed."""
-    path = os.path.join(os.path.dirname(S.__file__), "tuned", "splitk_mi355x_s60.txt")
+    path = os.path.join(os.path.dirname(S.__file__), "tuned", "splitk_mi355x.txt")
     for line in open(path):
         f = line.split()
         if len(f) == 4 and not line.startswith("#") and (int(f[0]), int(f[1]), int(f[2])) == (M, N, K):

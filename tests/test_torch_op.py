@@ -85,6 +85,29 @@ def test_bad_arguments_raise(ops):
         torch.ops.spmspm_amd.sparse_linear(x, layer.values, layer.bitmaps, layer.offsets, None, 192, 0, 0)
     with pytest.raises(RuntimeError):  # 24 columns: the library's unsupported-N error comes back as an exception
         layer(torch.zeros((24, 256), dtype=torch.float16, device="cuda"))
+    # operand types, devices and sizes are refused on the host, before any launch
+    op = torch.ops.spmspm_amd.sparse_linear
+    v, b, o = layer.values, layer.bitmaps, layer.offsets
+    with pytest.raises(ValueError, match="int32"):
+        op(x, v, b, o.long(), None, 128, 0, 0)
+    with pytest.raises(ValueError, match="int64"):
+        op(x, v, b.int(), o, None, 128, 0, 0)
+    with pytest.raises(ValueError, match="int16 or fp16"):
+        op(x, v.float(), b, o, None, 128, 0, 0)
+    with pytest.raises(ValueError, match="share x's device"):
+        op(x, v.cpu(), b, o, None, 128, 0, 0)
+    with pytest.raises(ValueError, match="share x's device"):
+        op(x, v, b.cpu(), o, None, 128, 0, 0)
+    with pytest.raises(ValueError, match="share x's device"):
+        op(x, v, b, o, torch.zeros(128, dtype=torch.float16), 128, 0, 0)
+    with pytest.raises(ValueError, match="contiguous"):
+        op(x, torch.stack([v, v], 1)[:, 0], b, o, None, 128, 0, 0)
+    with pytest.raises(ValueError, match="offsets end at"):
+        op(x, v[:-8], b, o, None, 128, 0, 0, layer.nnz)
+    with pytest.raises(ValueError, match="offsets end at"):
+        T.SparseLinearModule(128, 256, v[:-8], b, o)
+    y = op(x, v.view(torch.float16), b, o, None, 128, 0, 0, layer.nnz)  # fp16-typed values are the same bytes
+    assert torch.equal(y, layer(x))
 
 
 def _chain(T, comps, biases):
