@@ -33,7 +33,8 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=2000)
     p.add_argument("--warmup", type=int, default=100)
-    p.add_argument("--prewarm-ms", type=float, default=30.0, help="untimed calls before the warm-up steps (clock ramp)")
+    p.add_argument("--prewarm-ms", type=float, default=120.0,
+                   help="untimed calls before the warm-up steps: after idling, the first ~40 ms of calls run at ramping clocks")
     p.add_argument("--workload", default="opt30b_ffn1")
     p.add_argument("--n", type=int, default=None, help="override the workload's N")
     p.add_argument("--sparsity", type=float, default=None, help="override the workload's sparsity (0..1)")
@@ -50,6 +51,10 @@ def parse():
     p.add_argument("--chain-layers", type=int, default=40)
     p.add_argument("--no-stream-probe", action="store_true",
                    help="skip the read-stream probe (spmspm_amd/lib/stream_probe) behind roofline.stream_ceiling_gbs")
+    p.add_argument("--no-sweep", action="store_true",
+                   help="skip the sweep over the remaining benchmark cells (OPT-30B FFN1 at four sparsities x N = 8, "
+                        "16, 32; OPT-66B FFN2 at N = 64, 128; the other three OPT-13B linears)")
+    p.add_argument("--sweep-steps", type=int, default=200, help="timed calls per sweep cell")
     p.add_argument("--copy-probe", action="store_true",
                    help="also run three 256 MiB device-to-device copies (a known-size reference for HBM byte counters)")
     return p.parse_args()
@@ -179,6 +184,137 @@ def quick_measure(torch, S, hip, dev, workload, steps, warmup, seed):
             "main_kernel_gbs": algo / kern / 1e9, "main_kernel_roofline_frac": algo / kern / 1e9 / HBM_PEAK_GBS,
             "algorithmic_bytes": int(algo), "dense_fp16_us": td * 1e6, "speedup_vs_dense": td / wall,
             "rel_l2": float(np.linalg.norm(got - ref) / np.linalg.norm(ref))}
+
+
+def shader_clock_mhz(torch, L, side, burst):
+    """Shader clock while `burst` (a function issuing SpMM calls on the current stream for a few milliseconds) runs:
+    one idling wave on a second stream compares the shader-clock counter with the constant 100 MHz counter
+    (SpMM_ShaderClockProbe) for 2 ms of that time."""
+    ticks = torch.zeros(2, dtype=torch.int64, device="cuda:0")
+    torch.cuda.synchronize()
+    burst(20)  # the load is already running when the probe starts
+    if L.SpMM_ShaderClockProbe(side.cuda_stream, ticks.data_ptr(), 2000) != 0:
+        return None
+    burst(120)
+    torch.cuda.synchronize()
+    c, r = (int(v) for v in ticks.cpu())
+    return 100.0 * c / r if r > 0 else None
+
+
+def device_weights(torch, M, K, sparsity, pruning, seed, dev):
+    """Seeded synthetic weights made on the GPU (the host generator takes seconds per matrix of this size): fp16
+    N(0, 0.02), pruned with a uniform random mask or by magnitude over the whole matrix."""
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    W = torch.empty((M, K), dtype=torch.float16, device=dev)
+    rows = max(1, (1 << 25) // K)
+    for r0 in range(0, M, rows):
+        r1 = min(M, r0 + rows)
+        W[r0:r1] = (torch.randn((r1 - r0, K), generator=g, device=dev) * 0.02).to(torch.float16)
+    if pruning == "random":
+        for r0 in range(0, M, rows):
+            r1 = min(M, r0 + rows)
+            W[r0:r1][torch.rand((r1 - r0, K), generator=g, device=dev) < sparsity] = 0
+    else:
+        mag = W.abs().float().reshape(-1)
+        kth = int(round(sparsity * mag.numel()))
+        if kth > 0:
+            thresh = torch.kthvalue(mag, kth).values
+            W[W.abs().float() <= thresh] = 0
+        del mag
+    return W
+
+
+class SweepMatrix:
+    """One synthetic weight matrix of the sweep, generated and encoded on the device (the device encoder's arrays
+    are the host encoder's, bit for bit: tests/test_encoder_gpu.py), with enough resident copies that successive
+    calls cannot be served from the last-level cache."""
+
+    def __init__(self, torch, S, dev, M, K, sparsity, pruning, seed):
+        self.M, self.K, self.sparsity, self.pruning = M, K, sparsity, pruning
+        self.W = device_weights(torch, M, K, sparsity, pruning, seed, dev)
+        v, b, o = S.InitSparseMatrixA_bitmap_device(self.W)
+        self.nnz = int(v.numel())
+        self.fixed_bytes = 2 * self.nnz + 8 * b.numel() + 4 * o.numel()
+        copies = max(2, -(-3 * LLC_BYTES // self.fixed_bytes))
+        self.arrays = [(v, b, o)] + [(v.clone(), b.clone(), o.clone()) for _ in range(copies - 1)]
+
+
+def sweep_cell(torch, S, hip, dev, mat, N, steps, seed, name):
+    """One cell of the benchmark grid (the reference harness appends one CSV row per cell,
+    kernel_benchmark/spmm_test_utils.h:249-290): whole-call and main-kernel time, roofline fractions, result check."""
+    M, K = mat.M, mat.K
+    L = S.library()
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed + 77)
+    x = (torch.rand((N, K), generator=g, device=dev) * 2 - 1).to(torch.float16)
+    out = torch.empty((N, M), dtype=torch.float16, device=dev)
+    sk = S.SpMM_SplitK_Auto(M, N, K)
+    need = S.SpMM_WorkspaceBytes(M, N, K, sk)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream()
+    copies = len(mat.arrays)
+
+    def call(i):
+        v, b, o = mat.arrays[i % copies]
+        err = S.SpMM_SplitK_API(stream, v, b, o, x, out, M, N, K, ws, sk)
+        if err != 0:
+            raise RuntimeError(f"sweep cell {name}: hipError_t {err}")
+
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.02:  # clock ramp
+        for i in range(50):
+            call(i)
+        torch.cuda.synchronize()
+    g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    g0.record(stream)
+    for i in range(steps):
+        call(i)
+    g1.record(stream)
+    torch.cuda.synchronize()
+    call_s = g0.elapsed_time(g1) / 1e3 / steps
+    events = [(hip.event(), hip.event()) for _ in range(steps)]
+    for i in range(steps):
+        L.SpMM_TimeNextCall(events[i][0], events[i][1])
+        call(i)
+    torch.cuda.synchronize()
+    kern_s = float(np.mean([hip.elapsed_ms(e0, e1) for e0, e1 in events])) / 1e3
+    for e0, e1 in events:
+        hip.rt.hipEventDestroy(e0), hip.rt.hipEventDestroy(e1)
+    # result check: 64 sampled rows against a float64 product of the dense weights on the device
+    rows = torch.from_numpy(np.random.default_rng(3).choice(M, 64, replace=False)).to(dev)
+    ref = x.double() @ mat.W[rows].double().t()
+    got = out[:, rows].double()
+    rel_l2 = float((got - ref).norm() / ref.norm())
+    max_frac = float((got - ref).abs().max() / ref.abs().max())
+    if not (rel_l2 <= 1e-3 and max_frac <= 1e-2):
+        raise RuntimeError(f"sweep cell {name}: outside the tolerance (rel-L2 {rel_l2:.2e}, max {max_frac:.2e})")
+    algo = mat.fixed_bytes + 2 * K * N + 2 * M * N
+    flops = 2.0 * M * N * K
+    return {"cell": name, "M": M, "K": K, "N": N, "sparsity": mat.sparsity, "pruning": mat.pruning, "split_k": sk,
+            "kernel": L.SpMM_KernelName(M, N, K, sk).decode(), "us_per_call": call_s * 1e6,
+            "main_kernel_us": kern_s * 1e6, "roofline_frac": algo / call_s / 1e9 / HBM_PEAK_GBS,
+            "main_kernel_roofline_frac": algo / kern_s / 1e9 / HBM_PEAK_GBS, "tflops": flops / call_s / 1e12,
+            "algorithmic_bytes": int(algo), "rel_l2": rel_l2}
+
+
+def sweep(torch, S, hip, dev, steps, seed):
+    """The benchmark grid beyond the headline cell, each cell timed like the headline (GPU time of whole calls
+    back to back from stream events; the main kernel from events on its dispatches)."""
+    cells = []
+    grid = [("opt30b_ffn1", 28672, 7168, s, "random", (8, 16, 32)) for s in (0.4, 0.5, 0.6, 0.7)]
+    grid += [("opt66b_ffn2", 9216, 36864, 0.4, "random", (64, 128))]
+    grid += [("opt13b_out", 5120, 5120, 0.6, "magnitude", (16,)), ("opt13b_ffn1", 20480, 5120, 0.6, "magnitude", (16,)),
+             ("opt13b_ffn2", 5120, 20480, 0.6, "magnitude", (16,))]
+    for nm, M, K, sp, pruning, widths in grid:
+        mat = SweepMatrix(torch, S, dev, M, K, sp, pruning, seed)
+        for N in widths:
+            cells.append(sweep_cell(torch, S, hip, dev, mat, N, steps, seed, f"{nm}_s{int(round(sp * 100))}_n{N}"))
+        del mat
+        torch.cuda.empty_cache()
+    return {"steps_per_cell": steps, "cells": cells,
+            "what": "weights generated and encoded on the GPU (seeded); us_per_call = GPU time of whole calls (main "
+                    "kernel + split-K reduction) back to back; roofline_frac = algorithmic bytes / that time / 8 TB/s"}
 
 
 def device_encoder(torch, S, dev, W, comp, host_encode_s):
@@ -349,8 +485,9 @@ def main():
             L.SpMM_TimeNextCall(ev[0], ev[1])
         layers[j](xs[j], out=outs[j], stream=stream)
 
-    # The first ~100 calls after the GPU has been idle run 15-20 % slower (clocks ramping up); keep it busy for a
-    # moment before the W warm-up steps so that a short run measures the same machine state as a long one.
+    # The first ~40 ms of calls after the GPU has been idle run 10-15 % slower (clocks ramping up: 43 us per call
+    # falling to 38 us); keep it busy for a moment before the W warm-up steps so that a short run measures the same
+    # machine state as a long one.  The shader clock read below (1.9-2.3 GHz under this load) says which state that was.
     t0 = time.perf_counter()
     while time.perf_counter() - t0 < a.prewarm_ms * 1e-3:
         for i in range(50):
@@ -359,6 +496,13 @@ def main():
     for i in range(a.warmup):
         step(i)
     torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+
+    def burst(n):
+        for i in range(n):
+            step(i)
+
+    clock_before = shader_clock_mhz(torch, L, side, burst)
 
     # timed region 1: K steps, wall clock between synchronisations -> value; the same steps on the GPU's clock
     # (events recorded on the launch stream before the first and after the last call) -> roofline
@@ -380,6 +524,8 @@ def main():
     kern_ms = np.array([hip.elapsed_ms(e0, e1) for e0, e1 in events])
     for e0, e1 in events:
         hip.rt.hipEventDestroy(e0), hip.rt.hipEventDestroy(e1)
+
+    clock_after = shader_clock_mhz(torch, L, side, burst)
 
     if a.copy_probe:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
@@ -462,6 +608,12 @@ def main():
                                      "frac": achieved_main / HBM_PEAK_GBS,
                                      "timing": "HIP events attached to each main-kernel dispatch (kernel begin/end "
                                                "timestamps), the same K steps repeated after the first region"},
+                     "shader_clock_mhz": {"before": clock_before, "after": clock_after,
+                                          "what": "shader-clock counter against the 100 MHz counter over 2 ms of "
+                                                  "the same calls, one idling wave on a second stream "
+                                                  "(SpMM_ShaderClockProbe), before and after the timed regions"},
+                     "main_kernel_cycles_per_group_tile_and_cu":
+                         None if not clock_after else kern_avg_s * clock_after * 1e6 / ((M // 64) * (K // 64) / 256.0),
                      "stream_ceiling_gbs": None if stream_ceiling is None else stream_ceiling["stream_ceiling_gbs"],
                      "frac_of_stream_ceiling": None if stream_ceiling is None
                      else achieved / stream_ceiling["stream_ceiling_gbs"],
@@ -476,8 +628,13 @@ def main():
         out["opt13b_qkv"] = quick_measure(torch, S, hip, dev, "opt13b_qkv", max(20, a.steps // 2), a.warmup, a.seed)
     if not a.no_encoder:
         out["device_encoder"] = device_encoder(torch, S, dev, W, comp, t_enc)
-    if not a.no_chain:
+    if not a.no_sweep:
         del layers, xs, outs
+        layers = xs = outs = None
+        torch.cuda.empty_cache()
+        out["sweep"] = sweep(torch, S, hip, dev, a.sweep_steps, a.seed)
+    if not a.no_chain:
+        layers = xs = outs = None
         torch.cuda.empty_cache()
         out["decode_chain_opt13b"] = decode_chain(torch, S, dev, a.chain_layers, a.seed)
     if not a.no_cpu_baseline:

@@ -263,6 +263,15 @@ void SpMM_FreeWeights(void* values_d, int* offsets_d, int* median_d, uint64_t* b
 void SpMM_TimeNextCall(hipEvent_t before_main, hipEvent_t after_main);
 
 /*
+ * Reporting aid with no counterpart in the reference: launches one wave on `stream` that idles for about `spin_us`
+ * microseconds (1..100000) and writes two 64-bit counts to `ticks_d` (device memory, 16 bytes): by how much the
+ * shader-clock counter and the constant 100 MHz counter advanced meanwhile.  100 * ticks_d[0] / ticks_d[1] is the
+ * shader clock in MHz during that time; run on a second stream beside SpMM calls it is the clock those calls run
+ * at, which lets timings taken on different machines be compared in cycles.  Returns the launch status.
+ */
+int SpMM_ShaderClockProbe(hipStream_t stream, unsigned long long* ticks_d, int spin_us);
+
+/*
  * Name of the main kernel a call of SpMM_SplitK_API, SpMM_SplitK_API_Sized or SpMM_SplitK_API_NoAlloc with these
  * dimensions dispatches, as a profiler prints it, e.g. "spmm::spmm_bitmap_rows<1, true>" (second template argument:
  * fp32 partial sums to the workspace, which these three entry points use whenever K is split).  It does not hold

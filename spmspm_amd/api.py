@@ -87,6 +87,8 @@ def library():
     L.SpMM_Version.restype = C.c_char_p
     L.SpMM_KernelName.restype = C.c_char_p
     L.SpMM_KernelName.argtypes = [C.c_int] * 4
+    L.SpMM_ShaderClockProbe.restype = C.c_int
+    L.SpMM_ShaderClockProbe.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
     L.SpMM_TimeNextCall.restype = None
     L.SpMM_TimeNextCall.argtypes = [C.c_void_p, C.c_void_p]
     _lib = L

@@ -592,6 +592,35 @@ extern "C" void SpMM_TimeNextCall(hipEvent_t before_main, hipEvent_t after_main)
     t_after_main  = after_main;
 }
 
+// ---- shader clock probe ---------------------------------------------------------------------------------------
+// One wave spins for about `spin_us` microseconds of the constant 100 MHz counter (s_memrealtime) and reports how
+// far the shader-clock counter (s_memtime) advanced meanwhile.  Launched on a second stream while SpMM calls run, it
+// reads the clock the kernels actually run at, which is what a kernel bound inside the CU follows.
+namespace {
+__global__ __launch_bounds__(64) void shader_clock_probe(unsigned long long* out, unsigned spin_ticks)
+{
+    const unsigned long long r0 = __builtin_amdgcn_s_memrealtime(), c0 = __builtin_readcyclecounter();
+    unsigned long long       r1 = r0;
+    for (unsigned i = 0; i < (1u << 22) && r1 - r0 < spin_ticks; ++i) { // bounded: every wave reaches the end
+        __builtin_amdgcn_s_sleep(8);
+        r1 = __builtin_amdgcn_s_memrealtime();
+    }
+    const unsigned long long c1 = __builtin_readcyclecounter();
+    if (threadIdx.x == 0) {
+        out[0] = c1 - c0;
+        out[1] = r1 - r0;
+    }
+}
+} // namespace
+
+extern "C" int SpMM_ShaderClockProbe(hipStream_t stream, unsigned long long* ticks_d, int spin_us)
+{
+    if (ticks_d == nullptr || spin_us <= 0 || spin_us > 100000)
+        return (int)hipErrorInvalidValue;
+    return (int)spmm::launch_kernel(shader_clock_probe, dim3(1, 1, 1), dim3(64, 1, 1), stream, nullptr, nullptr,
+                                    ticks_d, (unsigned)spin_us * 100u);
+}
+
 #ifdef SPMM_KEEP_VARIANTS
 // Test build only (not in the header): selects the comparison kernel for the calls that follow.
 extern "C" void SpMM_Debug_SetKernelVariant(int variant)

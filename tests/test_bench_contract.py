@@ -29,7 +29,7 @@ def test_traffic_records_are_consistent_and_say_what_they_were_taken_for():
 @pytest.mark.gpu
 def test_bench_line_has_the_contract_fields():
     p = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "10", "--warmup", "2",
-                        "--workload", "opt13b_out", "--cpu-seconds", "1", "--no-chain", "--no-qkv"],
+                        "--workload", "opt13b_out", "--cpu-seconds", "1", "--no-chain", "--no-qkv", "--no-sweep"],
                        capture_output=True, text=True, timeout=600)
     assert p.returncode == 0, p.stderr[-2000:]
     lines = [l for l in p.stdout.splitlines() if l.startswith("{")]
