@@ -22,6 +22,7 @@ HIPCC_FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared", "-fvisibility=default",
     *DEVICE_FLAGS,
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
+    "-Wno-inline-asm",  # the wide kernel's direct-to-LDS load names m0, which the compiler calls reserved
 ]
 
 
