@@ -567,6 +567,55 @@ def test_opt13b_two_layer_chain_against_oracle(torch, oracle):
         assert_spmm_close(x.cpu().numpy(), x_ref, f"layer {layer} chained output")
 
 
+def test_opt13b_decode_chain_at_full_depth(torch):
+    """The OPT-13B decode-step configuration at its stated depth: 40 layers x {QKV, out-proj, FFN1, FFN2} at N = 16,
+    60 % magnitude pruning, built the way the benchmark builds it (four encoded matrices, a resident copy of each per
+    layer: 11.8 GB of compressed weights), chained on one stream.  Every one of the 160 linears is checked on 64
+    sampled rows against a float64 product of the dense weights with the input that linear was actually given; the
+    attention result fed to the output projection differs from layer to layer, so no two layers compute the same."""
+    N, layers = 16, 40
+    dev = "cuda:0"
+    first, dense = [], []
+    for i, (name, M, K) in enumerate(OPT13B_LINEARS):
+        W = make_weight(M, K, 0.6, seed=900 + i, pruning="magnitude")
+        # keep activations of order one down the chain (see the two-layer test)
+        W = (W.astype(np.float32) * np.float32(1.0 / (0.02 * np.sqrt(0.4 * K)))).astype(np.float16)
+        first.append(S.SparseLinear(S.InitSparseMatrixA_bitmap(W), device=dev, split_k=0))
+        dense.append(torch.from_numpy(W.view(np.int16)).to(dev).view(torch.float16))
+        del W
+    chain = [[l if j == 0 else l.clone() for l in first] for j in range(layers)]
+    g = torch.Generator(device=dev)
+    g.manual_seed(4)
+    h = (torch.rand((N, 5120), generator=g, device=dev) * 2 - 1).half()
+    attn = [(torch.rand((N, 5120), generator=g, device=dev) * 2 - 1).half() for _ in range(layers)]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    got = []
+    with torch.cuda.stream(side):
+        x = h
+        for j, (lq, lo, l1, l2) in enumerate(chain):
+            q = lq(x, stream=side)
+            o = lo(attn[j], stream=side)
+            f = l1(o, stream=side)
+            x2 = l2(f, stream=side)
+            got.append(((x, q), (attn[j], o), (o, f), (f, x2)))
+            x = x2
+    side.synchronize()
+    rng = np.random.default_rng(8)
+    worst = 0.0
+    for j, pairs in enumerate(got):
+        for (name, M, K), Wd, (xin, y) in zip(OPT13B_LINEARS, dense, pairs):
+            rows = torch.from_numpy(rng.choice(M, 64, replace=False)).to(dev)
+            ref = xin.double() @ Wd[rows].double().t()
+            d = y[:, rows].double() - ref
+            assert torch.isfinite(y).all(), f"layer {j} {name}: non-finite output"
+            rel = float(d.norm() / ref.norm())
+            frac = float(d.abs().max() / ref.abs().max())
+            assert rel <= 1e-3 and frac <= 1e-2, f"layer {j} {name}: rel-L2 {rel:.2e}, max {frac:.2e}"
+            worst = max(worst, rel)
+    print(f"40-layer chain: worst rel-L2 over 160 linears {worst:.2e}", flush=True)
+
+
 def test_opt66b_ffn2_full_size_wide_batches(torch):
     """OPT-66B FFN2 9216x36864 at 40 % sparsity, N = 64 and 128 (the widest configuration of the benchmark set):
     sampled rows against float64, and the sum over all rows of every output column against the same sum taken
