@@ -333,7 +333,23 @@ def device_encoder(torch, S, dev, W, comp, host_encode_s):
     t = (time.perf_counter() - t0) / reps
     algo = 2 * W.size + 2 * comp.values.size + 8 * comp.bitmaps.size + 4 * comp.offsets.size
     moved = algo + 2 * W.size  # W is read twice
+    # the one-pass form (W read once; values into a buffer sized beforehand, here the worst case M*K)
+    room = torch.empty(W.size, dtype=torch.int16, device=dev)
+    v1, b1, o1 = S.InitSparseMatrixA_bitmap_device_onepass(Wd, values=room)
+    torch.cuda.synchronize()
+    same1 = (np.array_equal(o1.cpu().numpy(), comp.offsets) and np.array_equal(b1.cpu().numpy().view(np.uint64), comp.bitmaps)
+             and np.array_equal(v1.cpu().numpy().view(np.uint16), comp.values))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        S.InitSparseMatrixA_bitmap_device_onepass(Wd, values=room)
+    torch.cuda.synchronize()
+    t1 = (time.perf_counter() - t0) / reps
+    del room
     return {"ms": t * 1e3, "identical_to_host_encoder": bool(same), "algorithmic_bytes": int(algo),
+            "one_pass": {"ms": t1 * 1e3, "identical_to_host_encoder": bool(same1), "gbs_algorithmic": algo / t1 / 1e9,
+                         "frac_of_hbm_peak": algo / t1 / 1e9 / HBM_PEAK_GBS,
+                         "what": "SpMM_EncodeDevice_OnePass: W read once, offsets by look-back between workgroups; "
+                                 "wall time of the call incl. its scratch clear and the read-back of the count"},
             "gbs_algorithmic": algo / t / 1e9, "gbs_moved": moved / t / 1e9, "frac_of_hbm_peak": algo / t / 1e9 / HBM_PEAK_GBS,
             "host_encoder_ms": host_encode_s * 1e3, "host_threads": os.cpu_count(),
             "what": "dense fp16 W in HBM -> bitmaps, offsets, values in HBM; W read once = algorithmic, read twice = moved"}

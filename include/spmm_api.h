@@ -209,6 +209,22 @@ int SpMM_EncodeDevice_Bitmaps(hipStream_t stream, const void* W, int M, int K, u
 int SpMM_EncodeDevice_Values(hipStream_t stream, const void* W, int M, int K, const int* offsets, void* values);
 
 /*
+ * The device encoder in one pass over W (the two calls above read W twice): the same three arrays, bit for bit,
+ * from one kernel, for a caller that can give `values` room before the number of values is known.
+ *   values_capacity  halves `values` can hold; M*K always suffices.  offsets[G] is the number actually written.
+ *   scratch          SpMM_EncodeDevice_ScratchBytes(M, K) bytes of device memory, 8-byte aligned, contents
+ *                    irrelevant on entry (the call clears it).  After the call has finished, scratch's second
+ *                    32-bit word is 0 on success; bit 1 (value 2) says `values` was too small (bitmaps and offsets
+ *                    are complete, some runs were not written), bit 0 that a workgroup gave up waiting for its
+ *                    predecessors (nothing is valid then; not expected on a healthy device).
+ * Asynchronous on `stream`; returns the launch status, or 1 for M or K not a multiple of 64 or a missing or
+ * misaligned scratch.  No counterpart in the reference.
+ */
+size_t SpMM_EncodeDevice_ScratchBytes(int M, int K);
+int    SpMM_EncodeDevice_OnePass(hipStream_t stream, const void* W, int M, int K, uint64_t* bitmaps, int* offsets,
+                                 void* values, size_t values_capacity, void* scratch);
+
+/*
  * File-to-file encoder, replaces Our_GenSparseMatrixBinFile
  * (csrc/SpMM_API.cuh:243-320; called through ctypes at
  * end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:88-102).

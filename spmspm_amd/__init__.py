@@ -8,6 +8,7 @@ from .api import (  # noqa: F401
     CompressedMatrix,
     InitSparseMatrixA_bitmap,
     InitSparseMatrixA_bitmap_device,
+    InitSparseMatrixA_bitmap_device_onepass,
     Our_GenSparseMatrixBinFile,
     SparseLinear,
     ACT_GELU,

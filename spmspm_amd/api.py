@@ -79,6 +79,11 @@ def library():
     L.SpMM_EncodeDevice_Bitmaps.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     L.SpMM_EncodeDevice_Values.restype = C.c_int
     L.SpMM_EncodeDevice_Values.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    L.SpMM_EncodeDevice_ScratchBytes.restype = C.c_size_t
+    L.SpMM_EncodeDevice_ScratchBytes.argtypes = [C.c_int, C.c_int]
+    L.SpMM_EncodeDevice_OnePass.restype = C.c_int
+    L.SpMM_EncodeDevice_OnePass.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                            C.c_size_t, C.c_void_p]
     L.InitSparseMatrixA_bitmap.restype = C.c_int
     L.InitSparseMatrixA_bitmap.argtypes = [C.c_void_p] + [C.c_int] * 8 + [
         C.POINTER(_u16p), C.POINTER(_i32p), C.POINTER(_i32p), C.POINTER(_i32p), C.POINTER(_u64p), _i32p]
@@ -353,6 +358,41 @@ def InitSparseMatrixA_bitmap_device(W, stream=None):
     if err != HIP_SUCCESS:
         raise RuntimeError(f"SpMM_EncodeDevice_Values failed with hipError_t {err}")
     return values[:n] if n else values[:0], bitmaps, offsets
+
+
+def InitSparseMatrixA_bitmap_device_onepass(W, capacity=None, stream=None, values=None):
+    """The device encoder in one pass over W (SpMM_EncodeDevice_OnePass): same arrays as
+    InitSparseMatrixA_bitmap_device.  `values` needs room before the count is known: `capacity` halves (default M*K,
+    which always suffices) are allocated, or a caller's int16 tensor `values` is used, and the result is a view of
+    the first offsets[G] of them.  Synchronises once to read the count and the kernel's status word."""
+    import torch
+    if W.dtype != torch.float16 or W.dim() != 2 or not W.is_contiguous() or not W.is_cuda:
+        raise ValueError("W must be a contiguous [M][K] fp16 tensor on the device")
+    M, K = W.shape
+    if M % 64 or K % 64:
+        raise ValueError("M and K must be multiples of 64")
+    G = (M // 64) * (K // 64)
+    L = library()
+    if values is None:
+        values = torch.empty(max(int(capacity if capacity is not None else M * K), 8), dtype=torch.int16, device=W.device)
+    elif values.dtype != torch.int16 or not values.is_contiguous() or values.device != W.device:
+        raise ValueError("values must be a contiguous int16 tensor on W's device")
+    bitmaps = torch.empty(64 * G, dtype=torch.int64, device=W.device)
+    offsets = torch.empty(G + 1, dtype=torch.int32, device=W.device)
+    scratch = torch.empty(L.SpMM_EncodeDevice_ScratchBytes(M, K) // 8 + 1, dtype=torch.int64, device=W.device)
+    err = L.SpMM_EncodeDevice_OnePass(_stream_handle(stream), _ptr(W), M, K, _ptr(bitmaps), _ptr(offsets),
+                                      _ptr(values), values.numel(), _ptr(scratch))
+    if err != HIP_SUCCESS:
+        raise RuntimeError(f"SpMM_EncodeDevice_OnePass failed with hipError_t {err}")
+    if stream is not None:
+        stream.synchronize()
+    status = int(scratch.view(torch.int32)[1].item())
+    n = int(offsets[-1].item())
+    if status & 1:
+        raise RuntimeError("SpMM_EncodeDevice_OnePass: a workgroup gave up waiting for its predecessors")
+    if status & 2:
+        raise ValueError(f"SpMM_EncodeDevice_OnePass: values holds {values.numel()} halves, the matrix needs {n}")
+    return values[:n], bitmaps, offsets
 
 
 def SpMM_WorkspaceBytesBiasAct(M, N, K, Split_K):

@@ -219,6 +219,151 @@ __global__ __launch_bounds__(kThreads) void encode_values(const uint16_t* __rest
         reinterpret_cast<uint4*>(values + base)[i] = reinterpret_cast<const uint4*>(out)[i];
 }
 
+// ---- one pass over W ----------------------------------------------------------------------------------------------
+// The two-call form reads W twice because a group tile's values cannot be placed before the populations of all
+// earlier group tiles are known.  Here one kernel reads W once: a workgroup (four waves = four consecutive group
+// tiles, taken in the order the workgroups start) builds its bitmaps and compacts its values into LDS, publishes the
+// sum of its padded populations, and learns where its run begins by looking back over its predecessors' published
+// sums (decoupled look-back: each predecessor shows either its own sum or, once it knows it, the sum of everything
+// up to and including itself, so a workgroup never waits for more than the nearest predecessors still at work).
+// Status words are 64 bits, {state, sum}, written and read whole with device-scope relaxed atomics: the word carries
+// everything its reader needs, so no fence (which on this part would write back a whole L2) is involved.
+// A workgroup only ever waits for workgroups that started before it and are therefore resident; the wait is bounded
+// all the same, and a workgroup that gives up sets an error word and ends normally.
+//
+// Measured on 28672 x 7168 at 70 % sparsity: 189 us against 179 us for the two passes together (74 + 91 + 15 us),
+// although only 561 MB cross the memory interface instead of 972 MB.  A workgroup's 32 KB of W are read in about the
+// time one trip to another workgroup's status word takes, so the look-back is not hidden behind work: persistent
+// workgroups that request their next rows of W before looking back (194 us), a window of 256 predecessors per trip
+// instead of 64 (283-302 us: four times the words to wait for), one polling lane instead of 64, and chunks dealt
+// round-robin without the ticket counter (220 us) all left it there or made it worse.  The call is kept for what it
+// saves in traffic and for callers that want one launch; the two-call form remains the faster one.
+constexpr unsigned kStateSum = 1, kStatePrefix = 2; // 0: nothing published yet
+constexpr unsigned kErrSpin = 1, kErrCapacity = 2;
+constexpr unsigned kSpinLimit = 1u << 16;
+
+struct OnePassHeader {
+    unsigned ticket, error, pad0, pad1;
+};
+
+__global__ __launch_bounds__(256) void zero_words(unsigned* p, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n)
+        p[i] = 0;
+}
+
+__device__ __forceinline__ unsigned long long status_load(const unsigned long long* p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void status_store(unsigned long long* p, unsigned state, unsigned sum)
+{
+    __hip_atomic_store(p, ((unsigned long long)state << 32) | sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__global__ __launch_bounds__(kThreads) void encode_onepass(const uint16_t* __restrict__ W, int K, int G,
+                                                           uint64_t* __restrict__ bitmaps, int* __restrict__ offsets,
+                                                           uint16_t* __restrict__ values, unsigned long long capacity,
+                                                           OnePassHeader* __restrict__ head,
+                                                           unsigned long long* __restrict__ status)
+{
+    __shared__ __attribute__((aligned(16))) uint16_t stage[kWavesPerWG][4096 + 8];
+    __shared__ unsigned s_vid, s_excl;
+    __shared__ int      s_count[kWavesPerWG];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (threadIdx.x == 0)
+        s_vid = __hip_atomic_fetch_add(&head->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const unsigned vid    = s_vid; // position of this workgroup in start order = its chunk of four group tiles
+    const long     g      = (long)vid * kWavesPerWG + wave;
+    const bool     active = g < G;
+    int            padded = 0;
+    uint16_t*      out    = stage[wave];
+    if (active) {
+        const LaneTile t = load_lane_tile(W, K, (int)g, lane);
+        bitmaps[(size_t)g * 64 + lane] = ((uint64_t)t.hi << 32) | t.lo;
+        const int pc    = __builtin_popcount(t.lo) + __builtin_popcount(t.hi);
+        const int inc   = wave_inclusive_scan(pc);
+        const int total = __builtin_amdgcn_readlane(inc, 63);
+        int       p     = inc - pc;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const unsigned bits = ((r < 4 ? t.lo : t.hi) >> (8 * (r & 3))) & 0xffu;
+            const unsigned d[4] = {t.row[r].x, t.row[r].y, t.row[r].z, t.row[r].w};
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+                if (bits & (1u << c))
+                    out[p++] = (uint16_t)(d[c >> 1] >> (16 * (c & 1)));
+        }
+        padded = (total + 7) & ~7;
+        if (lane < padded - total)
+            out[total + lane] = 0;
+    }
+    if (lane == 0)
+        s_count[wave] = padded;
+    __syncthreads();
+    unsigned agg = 0, before = 0;
+#pragma unroll
+    for (int w = 0; w < kWavesPerWG; ++w) {
+        agg += (unsigned)s_count[w];
+        before += w < wave ? (unsigned)s_count[w] : 0u;
+    }
+    if (wave == 0) {
+        if (lane == 0)
+            status_store(status + vid, vid == 0 ? kStatePrefix : kStateSum, agg);
+        unsigned excl = 0;
+        if (vid > 0) {
+            long     j     = (long)vid - 1;
+            unsigned spins = 0;
+            for (;;) {
+                const long               idx = j - lane; // lane 0 looks at the nearest predecessor
+                // in front of the first chunk lies a prefix of zero
+                const unsigned long long s   = idx >= 0 ? status_load(status + idx) : ((unsigned long long)kStatePrefix << 32);
+                const unsigned           st  = (unsigned)(s >> 32);
+                const unsigned long long inval = __ballot(st == 0), pref = __ballot(st == kStatePrefix);
+                const int first_inval = inval ? __builtin_ctzll(inval) : 64;
+                const int first_pref  = pref ? __builtin_ctzll(pref) : 64;
+                if (first_inval < first_pref) { // a predecessor this side of the nearest prefix has not published yet
+                    if (++spins > kSpinLimit) {
+                        if (lane == 0)
+                            __hip_atomic_fetch_or(&head->error, kErrSpin, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(2);
+                    continue;
+                }
+                const int      upto    = first_pref < 64 ? first_pref : 63;
+                const unsigned contrib = lane <= upto ? (unsigned)s : 0u;
+                excl += (unsigned)__builtin_amdgcn_readlane(wave_inclusive_scan((int)contrib), 63);
+                if (first_pref < 64)
+                    break;
+                j -= 64;
+            }
+            if (lane == 0)
+                status_store(status + vid, kStatePrefix, excl + agg);
+        }
+        if (lane == 0)
+            s_excl = excl;
+    }
+    __syncthreads();
+    if (!active)
+        return;
+    const unsigned long long base = (unsigned long long)s_excl + before;
+    if (lane == 0) {
+        offsets[g + 1] = (int)(base + (unsigned)padded);
+        if (g == 0)
+            offsets[0] = 0;
+    }
+    if (base + (unsigned)padded > capacity) {
+        if (lane == 0)
+            __hip_atomic_fetch_or(&head->error, kErrCapacity, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+    for (int i = lane; i < (padded >> 3); i += 64)
+        reinterpret_cast<uint4*>(values + base)[i] = reinterpret_cast<const uint4*>(out)[i];
+}
+
 inline int check(int M, int K)
 {
     if (M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0) {
@@ -260,5 +405,34 @@ extern "C" int SpMM_EncodeDevice_Values(hipStream_t stream, const void* W, int M
     dim3 grid((unsigned)((G + spmm_enc::kWavesPerWG - 1) / spmm_enc::kWavesPerWG), 1, 1);
     hipLaunchKernelGGL(spmm_enc::encode_values, grid, dim3(spmm_enc::kThreads, 1, 1), 0, stream,
                        static_cast<const uint16_t*>(W), K, G, offsets, static_cast<uint16_t*>(values));
+    return (int)hipGetLastError();
+}
+
+extern "C" size_t SpMM_EncodeDevice_ScratchBytes(int M, int K)
+{
+    if (M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
+        return 0;
+    const size_t G = (size_t)(M / 64) * (size_t)(K / 64);
+    return sizeof(spmm_enc::OnePassHeader) + 8 * ((G + spmm_enc::kWavesPerWG - 1) / spmm_enc::kWavesPerWG);
+}
+
+extern "C" int SpMM_EncodeDevice_OnePass(hipStream_t stream, const void* W, int M, int K, uint64_t* bitmaps,
+                                         int* offsets, void* values, size_t values_capacity, void* scratch)
+{
+    if (int e = spmm_enc::check(M, K))
+        return e;
+    if (scratch == nullptr || (reinterpret_cast<uintptr_t>(scratch) & 7) != 0)
+        return (int)hipErrorInvalidValue;
+    const int    G      = (M / 64) * (K / 64);
+    const size_t chunks = ((size_t)G + spmm_enc::kWavesPerWG - 1) / spmm_enc::kWavesPerWG;
+    const size_t words  = SpMM_EncodeDevice_ScratchBytes(M, K) / 4;
+    (void)hipGetLastError();
+    hipLaunchKernelGGL(spmm_enc::zero_words, dim3((unsigned)((words + 255) / 256), 1, 1), dim3(256, 1, 1), 0, stream,
+                       static_cast<unsigned*>(scratch), words);
+    auto* head   = static_cast<spmm_enc::OnePassHeader*>(scratch);
+    auto* status = reinterpret_cast<unsigned long long*>(head + 1);
+    hipLaunchKernelGGL(spmm_enc::encode_onepass, dim3((unsigned)chunks, 1, 1), dim3(spmm_enc::kThreads, 1, 1), 0, stream,
+                       static_cast<const uint16_t*>(W), K, G, bitmaps, offsets, static_cast<uint16_t*>(values),
+                       (unsigned long long)values_capacity, head, status);
     return (int)hipGetLastError();
 }

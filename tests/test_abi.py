@@ -24,7 +24,8 @@ def test_header_declares_the_expected_entry_points():
               "SpMM_EncodeDevice_Values", "SpMM_SplitK_TableSet", "SpMM_SplitK_TableLoad", "SpMM_SplitK_TableSave",
               "SpMM_SplitK_TableClear", "SpMM_SplitK_API_NoAlloc", "SpMM_SplitK_API_Sized", "SpMM_KernelName",
               "SpMM_SplitK_TableSetMany", "SpMM_SplitK_CostModel", "SpMM_SplitK_AutoNoAlloc", "SpMM_ReadWeightFiles",
-              "SpMM_LoadWeightFiles", "SpMM_FreeWeights", "SpMM_ShaderClockProbe"):
+              "SpMM_LoadWeightFiles", "SpMM_FreeWeights", "SpMM_ShaderClockProbe",
+              "SpMM_EncodeDevice_OnePass", "SpMM_EncodeDevice_ScratchBytes"):
         assert n in names
 
 

@@ -71,6 +71,56 @@ def test_device_encoder_reproduces_the_golden_encodings(torch, golden):
     assert ran >= 7
 
 
+@pytest.mark.parametrize("M,K,sparsity", [(64, 64, 0.5), (128, 192, 0.7), (512, 1024, 0.9), (1024, 256, 0.0),
+                                          (256, 256, 1.0), (2048, 4096, 0.6), (65536, 64, 0.5), (64 * 37, 64 * 61, 0.8)])
+def test_one_pass_device_encoder_is_bit_identical_to_the_oracle(torch, oracle, M, K, sparsity):
+    """SpMM_EncodeDevice_OnePass (W read once, offsets by look-back between workgroups) against the oracle; the last
+    shape has 2257 group tiles = 565 workgroups, so the look-back spans several windows of 64 predecessors."""
+    W = _special_matrix(M, K, seed=M + K) if (M >= 192 and K >= 128) else make_weight(M, K, sparsity, seed=M + K)
+    if sparsity == 1.0:
+        W[:] = 0
+    want = oracle.encode(W, M, K)
+    Wd = torch.from_numpy(W.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+    print(f"one-pass case M={M} K={K} s={sparsity}", flush=True)
+    for rep in range(2):  # the second run finds the scratch and output buffers of the first in the allocator
+        values, bitmaps, offsets = S.InitSparseMatrixA_bitmap_device_onepass(Wd)
+        torch.cuda.synchronize()
+        assert np.array_equal(offsets.cpu().numpy(), want["global"])
+        assert np.array_equal(bitmaps.cpu().numpy().view(np.uint64), want["bitmap"])
+        assert np.array_equal(values.cpu().numpy().view(np.uint16), want["values"])
+
+
+def test_one_pass_device_encoder_golden_and_capacity(torch, golden):
+    ran = 0
+    for name, case in golden.items():
+        W = case["W"]
+        M, K = W.shape
+        if M % 64 or K % 64:
+            continue
+        Wd = torch.from_numpy(W.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+        values, bitmaps, offsets = S.InitSparseMatrixA_bitmap_device_onepass(Wd)
+        torch.cuda.synchronize()
+        assert np.array_equal(offsets.cpu().numpy(), case["offsets"]), name
+        assert np.array_equal(bitmaps.cpu().numpy().view(np.uint64), case["bitmaps"]), name
+        assert np.array_equal(values.cpu().numpy().view(np.uint16), case["values"]), name
+        ran += 1
+    assert ran >= 7
+    # a values buffer that is too small: reported, nothing written past its end, bitmaps and offsets still complete
+    W = make_weight(256, 256, 0.5, seed=5)
+    comp = S.InitSparseMatrixA_bitmap(W)
+    Wd = torch.from_numpy(W.view(np.int16).copy()).to("cuda:0").view(torch.float16)
+    need = int(comp.offsets[-1])
+    buf = torch.full((need + 64,), 0x5a5a, dtype=torch.int16, device="cuda:0")
+    with pytest.raises(ValueError, match="the matrix needs %d" % need):
+        S.InitSparseMatrixA_bitmap_device_onepass(Wd, values=buf[:need - 8])
+    assert (buf[need - 8:] == 0x5a5a).all()
+    v, b, o = S.InitSparseMatrixA_bitmap_device_onepass(Wd, values=buf[:need])  # exactly enough
+    assert np.array_equal(v.cpu().numpy().view(np.uint16), comp.values) and (buf[need:] == 0x5a5a).all()
+    L = S.library()
+    assert L.SpMM_EncodeDevice_OnePass(None, Wd.data_ptr(), 256, 256, b.data_ptr(), o.data_ptr(), buf.data_ptr(), need, None) == 1
+    assert L.SpMM_EncodeDevice_ScratchBytes(256, 256) == 16 + 8 * 4 and L.SpMM_EncodeDevice_ScratchBytes(100, 64) == 0
+
+
 def test_device_encoded_weights_multiply_correctly(torch, oracle):
     M, K, N = 1024, 2048, 16
     W = make_weight(M, K, 0.7, seed=77)
