@@ -129,6 +129,27 @@ def cpu_baseline(comp, X, seconds):
     }
 
 
+def bound_call(L, layer, x, out, stream_handle):
+    """`SpMM_SplitK_API` on one resident weight copy with every argument converted beforehand: what a C caller's loop
+    costs per step.  (The Python convenience wrapper `SparseLinear.__call__` checks and converts its arguments on
+    every call, 20-40 us of host time per call on these boxes: more than the GPU needs for the smaller shapes, so a
+    loop over it measures the host.)"""
+    import ctypes as C
+    N = x.shape[0]
+    sk = layer._plan(N)[0]
+    ws = layer.workspace(N)
+    args = (C.c_void_p(stream_handle), C.c_void_p(layer.values.data_ptr()), C.c_void_p(layer.bitmaps.data_ptr()),
+            C.c_void_p(layer.offsets.data_ptr()), C.c_void_p(x.data_ptr()), C.c_void_p(out.data_ptr()),
+            C.c_int(layer.M), C.c_int(N), C.c_int(layer.K), C.c_void_p(ws.data_ptr() if ws is not None else None),
+            C.c_int(sk))
+    fn = L.SpMM_SplitK_API
+
+    def call():
+        if fn(*args):
+            raise RuntimeError("SpMM_SplitK_API failed")
+    return call
+
+
 def quick_measure(torch, S, hip, dev, workload, steps, warmup, seed):
     """The timing of main(), in short, for one more named workload: whole-call TFLOP/s, main-kernel GB/s and
     roofline fraction, and the dense fp16 product of the same shape in the same run."""
@@ -146,20 +167,19 @@ def quick_measure(torch, S, hip, dev, workload, steps, warmup, seed):
     out = torch.empty((N, M), dtype=torch.float16, device=dev)
     stream = torch.cuda.current_stream()
     L = S.library()
-    for l in layers:
-        l.workspace(N)
+    calls = [bound_call(L, l, x, out, stream.cuda_stream) for l in layers]
     for i in range(warmup):
-        layers[i % copies](x, out=out, stream=stream)
+        calls[i % copies]()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
-        layers[i % copies](x, out=out, stream=stream)
+        calls[i % copies]()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
     events = [(hip.event(), hip.event()) for _ in range(steps)]
     for i in range(steps):
         L.SpMM_TimeNextCall(events[i][0], events[i][1])
-        layers[i % copies](x, out=out, stream=stream)
+        calls[i % copies]()
     torch.cuda.synchronize()
     kern = float(np.mean([hip.elapsed_ms(e0, e1) for e0, e1 in events])) / 1e3
     for e0, e1 in events:
@@ -344,15 +364,44 @@ def device_encoder(torch, S, dev, W, comp, host_encode_s):
         S.InitSparseMatrixA_bitmap_device_onepass(Wd, values=room)
     torch.cuda.synchronize()
     t1 = (time.perf_counter() - t0) / reps
-    del room
-    return {"ms": t * 1e3, "identical_to_host_encoder": bool(same), "algorithmic_bytes": int(algo),
-            "one_pass": {"ms": t1 * 1e3, "identical_to_host_encoder": bool(same1), "gbs_algorithmic": algo / t1 / 1e9,
-                         "frac_of_hbm_peak": algo / t1 / 1e9 / HBM_PEAK_GBS,
-                         "what": "SpMM_EncodeDevice_OnePass: W read once, offsets by look-back between workgroups; "
-                                 "wall time of the call incl. its scratch clear and the read-back of the count"},
-            "gbs_algorithmic": algo / t / 1e9, "gbs_moved": moved / t / 1e9, "frac_of_hbm_peak": algo / t / 1e9 / HBM_PEAK_GBS,
+    # GPU time of the entry points alone, every buffer allocated beforehand: events on the stream around `reps` calls
+    L, M, K = S.library(), W.shape[0], W.shape[1]
+    scratch = torch.empty(L.SpMM_EncodeDevice_ScratchBytes(M, K) // 8 + 1, dtype=torch.int64, device=dev)
+    ptr = lambda x: x.data_ptr()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def gpu_us(call):
+        call()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
+
+    def two_calls():
+        assert L.SpMM_EncodeDevice_Bitmaps(stream, ptr(Wd), M, K, ptr(b1), ptr(o1)) == 0
+        assert L.SpMM_EncodeDevice_Values(stream, ptr(Wd), M, K, ptr(o1), ptr(room)) == 0
+
+    def one_call():
+        assert L.SpMM_EncodeDevice_OnePass(stream, ptr(Wd), M, K, ptr(b1), ptr(o1), ptr(room), room.numel(), ptr(scratch)) == 0
+
+    us2, us1 = gpu_us(two_calls), gpu_us(one_call)
+    del room, scratch
+    return {"ms": t * 1e3, "gpu_us": us2, "identical_to_host_encoder": bool(same), "algorithmic_bytes": int(algo),
+            "one_pass": {"ms": t1 * 1e3, "gpu_us": us1, "identical_to_host_encoder": bool(same1),
+                         "gbs_algorithmic": algo / us1 / 1e3, "frac_of_hbm_peak": algo / us1 / 1e3 / HBM_PEAK_GBS,
+                         "what": "SpMM_EncodeDevice_OnePass: W read once, offsets by look-back between workgroups; ms = "
+                                 "wall time of the Python call incl. its allocations, scratch clear and the read-back of "
+                                 "the count; gpu_us = GPU time of the entry point alone (stream events), which the rates "
+                                 "are taken from"},
+            "gbs_algorithmic": algo / us2 / 1e3, "gbs_moved": moved / us2 / 1e3, "frac_of_hbm_peak": algo / us2 / 1e3 / HBM_PEAK_GBS,
             "host_encoder_ms": host_encode_s * 1e3, "host_threads": os.cpu_count(),
-            "what": "dense fp16 W in HBM -> bitmaps, offsets, values in HBM; W read once = algorithmic, read twice = moved"}
+            "what": "dense fp16 W in HBM -> bitmaps, offsets, values in HBM; W read once = algorithmic, read twice = moved; "
+                    "ms = wall time of the Python call (two entry points, two allocations, the read-back of the count "
+                    "between them); gpu_us = GPU time of the two entry points back to back, which the rates are taken from"}
 
 
 def decode_chain(torch, S, dev, layers, seed):
@@ -495,11 +544,12 @@ def main():
     stream = torch.cuda.current_stream()
     shandle = stream.cuda_stream
 
+    calls = [bound_call(L, layers[j], xs[j], outs[j], shandle) for j in range(copies)]
+
     def step(i, ev=None):
-        j = i % copies
         if ev is not None:
             L.SpMM_TimeNextCall(ev[0], ev[1])
-        layers[j](xs[j], out=outs[j], stream=stream)
+        calls[i % copies]()
 
     # The first ~40 ms of calls after the GPU has been idle run 10-15 % slower (clocks ramping up: 43 us per call
     # falling to 38 us); keep it busy for a moment before the W warm-up steps so that a short run measures the same

