@@ -176,3 +176,49 @@ def test_device_encoder_offsets_scan_across_many_blocks(torch, oracle):
     torch.cuda.synchronize()
     assert np.array_equal(offsets.cpu().numpy(), comp.offsets)
     assert np.array_equal(values.cpu().numpy().view(np.uint16), comp.values)
+
+
+def test_weight_files_load_into_device_arrays_and_multiply(torch, oracle, tmp_path):
+    """SpMM_LoadWeightFiles: the six files Our_GenSparseMatrixBinFile writes -> device arrays equal to the oracle's
+    encoding, usable by the SpMM as they are; a damaged file leaves nothing behind."""
+    import ctypes as C
+    M, K, N = 256, 512, 16
+    W = make_weight(M, K, 0.6, seed=31)
+    X = make_activations(K, N, seed=31)
+    dense = tmp_path / "w.bin"
+    W.tofile(dense)
+    names = [str(tmp_path / n).encode() for n in ("v", "g", "m", "b", "x", "s")]
+    S.Our_GenSparseMatrixBinFile(str(dense), M, K, *[n.decode() for n in names])
+    L = S.library()
+    ptrs = [C.c_void_p() for _ in range(5)]
+    count = C.c_int(-1)
+    G = L.SpMM_LoadWeightFiles(*names, M, K, *[C.byref(p) for p in ptrs], C.byref(count))
+    want = oracle.encode(W, M, K)
+    assert G == (M // 64) * (K // 64) and count.value == int(want["global"][-1])
+    values_d, offsets_d, median_d, bitmaps_d, max_nnz_d = [p.value for p in ptrs]
+    assert all(p for p in (values_d, offsets_d, median_d, bitmaps_d, max_nnz_d))
+
+    def fetch(ptr, dtype, n):  # device -> host through a torch tensor of the same size
+        t = torch.empty(n, dtype=dtype, device="cuda:0")
+        hip = C.CDLL("libamdhip64.so")
+        hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        assert hip.hipMemcpy(t.data_ptr(), ptr, t.numel() * t.element_size(), 3) == 0  # device to device
+        return t.cpu().numpy()
+
+    assert np.array_equal(fetch(values_d, torch.int16, count.value).view(np.uint16), want["values"])
+    assert np.array_equal(fetch(offsets_d, torch.int32, G + 1), want["global"])
+    assert np.array_equal(fetch(bitmaps_d, torch.int64, 64 * G).view(np.uint64), want["bitmap"])
+    assert np.array_equal(fetch(median_d, torch.int32, 4 * G), want["median"])
+    x = torch.from_numpy(X.view(np.int16).copy()).to("cuda:0")
+    out = torch.empty((N, M), dtype=torch.int16, device="cuda:0")
+    ws = torch.empty(S.SpMM_WorkspaceBytes(M, N, K, 0) + 16, dtype=torch.uint8, device="cuda:0")
+    assert S.SpMM_SplitK_API(None, values_d, bitmaps_d, offsets_d, x, out, M, N, K, ws, 0) == 0
+    torch.cuda.synchronize()
+    assert_spmm_close(out.cpu().numpy().view(np.float16), X.astype(np.float64) @ W.astype(np.float64).T, "loaded weights")
+    L.SpMM_FreeWeights(*ptrs)
+    # a values file cut short: refused, the out-pointers stay as they were
+    with open(names[0].decode(), "r+b") as f:
+        f.truncate(10)
+    ptrs = [C.c_void_p() for _ in range(5)]
+    assert L.SpMM_LoadWeightFiles(*names, M, K, *[C.byref(p) for p in ptrs], None) == -1
+    assert all(p.value is None for p in ptrs)
