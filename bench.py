@@ -129,6 +129,18 @@ def cpu_baseline(comp, X, seconds):
     }
 
 
+def ramp(torch, issue, ms=40.0):
+    """Keeps the GPU busy for `ms` with `issue()` (a function that queues about a millisecond of work).  After any idle
+    of a few milliseconds (a host phase, the first use of a new stream, a read-back) the shader clock needs about
+    20 ms of load to come back, and calls in that window take 15-20 % longer (43 us falling to 36 us per call on the
+    target shape): every timed region below starts from a ramped clock, so a short run measures the same machine state
+    as a long one."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < ms * 1e-3:
+        issue()
+        torch.cuda.synchronize()
+
+
 def bound_call(L, layer, x, out, stream_handle):
     """`SpMM_SplitK_API` on one resident weight copy with every argument converted beforehand: what a C caller's loop
     costs per step.  (The Python convenience wrapper `SparseLinear.__call__` checks and converts its arguments on
@@ -168,6 +180,7 @@ def quick_measure(torch, S, hip, dev, workload, steps, warmup, seed):
     stream = torch.cuda.current_stream()
     L = S.library()
     calls = [bound_call(L, l, x, out, stream.cuda_stream) for l in layers]
+    ramp(torch, lambda: [calls[i % copies]() for i in range(40)])
     for i in range(warmup):
         calls[i % copies]()
     torch.cuda.synchronize()
@@ -189,9 +202,7 @@ def quick_measure(torch, S, hip, dev, workload, steps, warmup, seed):
     ref = X.astype(np.float64) @ W[rows].astype(np.float64).T
     Wd = [torch.from_numpy(W.view(np.int16)).to(dev).view(torch.float16)]
     Wd += [Wd[0].clone() for _ in range(max(2, -(-3 * LLC_BYTES // (2 * M * K))) - 1)]
-    for i in range(5):
-        torch.matmul(x, Wd[i % len(Wd)].t())
-    torch.cuda.synchronize()
+    ramp(torch, lambda: [torch.matmul(x, Wd[i % len(Wd)].t()) for i in range(30)])
     t0 = time.perf_counter()
     for i in range(steps):
         torch.matmul(x, Wd[i % len(Wd)].t())
@@ -281,11 +292,7 @@ def sweep_cell(torch, S, hip, dev, mat, N, steps, seed, name):
         if err != 0:
             raise RuntimeError(f"sweep cell {name}: hipError_t {err}")
 
-    t0 = time.perf_counter()
-    while time.perf_counter() - t0 < 0.02:  # clock ramp
-        for i in range(50):
-            call(i)
-        torch.cuda.synchronize()
+    ramp(torch, lambda: [call(i) for i in range(30)])
     g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     g0.record(stream)
     for i in range(steps):
@@ -371,8 +378,7 @@ def device_encoder(torch, S, dev, W, comp, host_encode_s):
     stream = torch.cuda.current_stream().cuda_stream
 
     def gpu_us(call):
-        call()
-        torch.cuda.synchronize()
+        ramp(torch, lambda: [call() for _ in range(5)])
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(reps):
@@ -451,8 +457,7 @@ def decode_chain(torch, S, dev, layers, seed):
             x = torch.matmul(f, w2.t(), out=hs[j & 1])
 
     def timed(fn, reps):
-        fn()
-        torch.cuda.synchronize()
+        ramp(torch, fn)
         t0 = time.perf_counter()
         for _ in range(reps):
             fn()
@@ -551,24 +556,20 @@ def main():
             L.SpMM_TimeNextCall(ev[0], ev[1])
         calls[i % copies]()
 
-    # The first ~40 ms of calls after the GPU has been idle run 10-15 % slower (clocks ramping up: 43 us per call
-    # falling to 38 us); keep it busy for a moment before the W warm-up steps so that a short run measures the same
-    # machine state as a long one.  The shader clock read below (1.9-2.3 GHz under this load) says which state that was.
-    t0 = time.perf_counter()
-    while time.perf_counter() - t0 < a.prewarm_ms * 1e-3:
-        for i in range(50):
-            step(i)
-        torch.cuda.synchronize()
-    for i in range(a.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    side = torch.cuda.Stream()
-
+    # Calls after the GPU has been idle run 15-20 % slower for about 20 ms (ramp()); keep it busy before the W warm-up
+    # steps.  The shader clock read below (1.9-2.3 GHz under this load) says which state the timed region saw.
     def burst(n):
         for i in range(n):
             step(i)
 
+    ramp(torch, lambda: burst(50), a.prewarm_ms)
+    side = torch.cuda.Stream()
     clock_before = shader_clock_mhz(torch, L, side, burst)
+    # the probe is the first use of a second stream, which idles the GPU for some milliseconds: ramp again
+    ramp(torch, lambda: burst(50), max(40.0, a.prewarm_ms / 2) if a.prewarm_ms > 0 else 0.0)
+    for i in range(a.warmup):
+        step(i)
+    torch.cuda.synchronize()
 
     # timed region 1: K steps, wall clock between synchronisations -> value; the same steps on the GPU's clock
     # (events recorded on the launch stream before the first and after the last call) -> roofline
@@ -618,9 +619,7 @@ def main():
     dense = None
     if not a.no_dense:
         Wd = [torch.from_numpy(W.view(np.int16)).to(dev).view(torch.float16) for _ in range(max(2, -(-3 * LLC_BYTES // (2 * M * K))))]
-        for i in range(5):
-            torch.matmul(xs[0], Wd[i % len(Wd)].t())
-        torch.cuda.synchronize()
+        ramp(torch, lambda: [torch.matmul(xs[0], Wd[i % len(Wd)].t()) for i in range(20)])
         t0 = time.perf_counter()
         reps = max(20, a.steps // 4)
         for i in range(reps):
