@@ -60,8 +60,12 @@ typedef struct ihipEvent_t*  hipEvent_t;
  * entry do not matter.
  * Returns a hipError_t value as int: 0 on success; 999 (hipErrorUnknown) with
  * the reference's message for an unsupported N (csrc/SpMM_API.cuh:91-94);
- * 1 (hipErrorInvalidValue) for M or K not a multiple of 64 or a missing
- * workspace; otherwise the launch status (csrc/SpMM_API.cuh:99-109).
+ * 1 (hipErrorInvalidValue) for M or K not a multiple of 64, a missing
+ * workspace, or a pointer that is NULL or not aligned as the kernels need
+ * (values, X, C and workspace 16 bytes, bitmaps 8, offsets 4: refused on the
+ * host, where the reference would fault on the device); otherwise the launch
+ * status (csrc/SpMM_API.cuh:99-109).  The same holds for the other SpMM
+ * entry points below.
  */
 int SpMM_SplitK_API(hipStream_t stream, const void* values, const uint64_t* bitmaps, const int* offsets,
                     const void* X, void* C, int M, int N, int K, void* workspace, int Split_K);

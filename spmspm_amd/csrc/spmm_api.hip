@@ -267,6 +267,16 @@ int run(hipStream_t stream, const void* values, const uint64_t* bitmaps, const i
         std::fflush(stdout);
         return (int)hipErrorInvalidValue;
     }
+    // The kernels read and write 16 bytes at a time (8 for bitmaps): an address they cannot use is refused here, on the
+    // host; on the device it would be a memory fault.
+    const auto bad = [](const void* p, uintptr_t align) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & (align - 1)) != 0; };
+    if (bad(values, 16) || bad(bitmaps, 8) || bad(offsets, 4) || bad(X, 16) || bad(C, 16) ||
+        (workspace != nullptr && bad(workspace, 16)) || (bias != nullptr && bad(bias, 2))) {
+        std::printf("MM_Sparse_API Error: a null or misaligned device pointer (values, X, C and workspace: 16 bytes, "
+                    "bitmaps: 8, offsets: 4)!\n");
+        std::fflush(stdout);
+        return (int)hipErrorInvalidValue;
+    }
     hipError_t err = spmm::launch_spmm(stream, static_cast<const __half*>(values), bitmaps, offsets,
                                        static_cast<const __half*>(X), static_cast<__half*>(C), M, N, K, workspace,
                                        split_k, fp32_partials, before, after, epilogue);

@@ -216,6 +216,21 @@ def test_tuner_candidates_and_presets():
     assert (28672, 7168) in tuner.PRESETS["opt30b"] and len(tuner.PRESETS["opt13b"]) == 4
 
 
+def test_null_and_misaligned_pointers_are_refused_on_the_host(capfd):
+    """Addresses the kernels cannot use (null, or off the 16-byte grid their loads and stores assume) never reach the
+    device: every entry point returns hipErrorInvalidValue before it launches anything."""
+    a = 1 << 20  # a plausible, aligned, never dereferenced address
+    ok = dict(values=a, bitmaps=a, offsets=a, X=a, C=a)
+    for name, bad in (("values", 0), ("values", a + 2), ("bitmaps", a + 4), ("offsets", a + 2), ("X", a + 8), ("C", a + 4), ("X", 0)):
+        p = dict(ok, **{name: bad})
+        capfd.readouterr()
+        assert S.SpMM_SplitK_API(0, p["values"], p["bitmaps"], p["offsets"], p["X"], p["C"], 64, 16, 64, 0, 1) == 1, name
+        assert "null or misaligned" in capfd.readouterr().out
+        assert S.SpMM_SplitK_API_NoAlloc(0, p["values"], p["bitmaps"], p["offsets"], p["X"], p["C"], 64, 16, 64, 1) == 1
+    assert S.SpMM_SplitK_API(0, a, a, a, a, a, 128, 16, 128, a + 4, 2) == 1  # a workspace off the grid
+    assert S.SpMM_SplitK_API_BiasAct(0, a, a, a, a, a, 64, 16, 64, a, 1, a + 1, 0) == 1  # an odd bias address
+
+
 def test_sized_entry_point_refuses_a_small_workspace_without_a_gpu(capfd):
     """The size check comes before anything touches the device: a too-small workspace returns
     hipErrorInvalidValue for an explicit split and for the library's own choice, also after the table has changed
