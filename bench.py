@@ -44,7 +44,7 @@ def parse():
     p.add_argument("--no-dense", action="store_true")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     p.add_argument("--no-qkv", action="store_true",
-                   help="skip the short extra measurement of the OPT-13B fused-QKV shape (BASELINE configs[1])")
+                   help="skip the short extra measurement of the OPT-13B fused-QKV shape (the 15360x5120 decode linear)")
     p.add_argument("--no-encoder", action="store_true", help="skip timing the device encoder on the workload's W")
     p.add_argument("--no-chain", action="store_true",
                    help="skip the OPT-13B decode-step chain (40 layers x 4 linears, sparse vs dense, same run)")

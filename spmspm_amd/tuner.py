@@ -18,7 +18,7 @@ import numpy as np
 from . import api as A
 from .synthetic import make_activations, make_weight
 
-# (M, K) of the decode-step linears, as in BASELINE's configurations
+# (M, K) of the decode-step linears of the benchmark configurations
 PRESETS = {
     "opt13b": [(15360, 5120), (5120, 5120), (20480, 5120), (5120, 20480)],
     "opt30b": [(21504, 7168), (7168, 7168), (28672, 7168), (7168, 28672)],
