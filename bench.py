@@ -562,11 +562,13 @@ def main():
         for i in range(n):
             step(i)
 
-    ramp(torch, lambda: burst(50), a.prewarm_ms)
+    # The first use of a second stream idles the GPU for some milliseconds (its queue is set up): do it now, with a
+    # throw-away probe, so that the probe before the timed region reads a ramped clock and leaves no gap behind it.
     side = torch.cuda.Stream()
+    shader_clock_mhz(torch, L, side, burst)
+    ramp(torch, lambda: burst(50), a.prewarm_ms)
     clock_before = shader_clock_mhz(torch, L, side, burst)
-    # the probe is the first use of a second stream, which idles the GPU for some milliseconds: ramp again
-    ramp(torch, lambda: burst(50), max(40.0, a.prewarm_ms / 2) if a.prewarm_ms > 0 else 0.0)
+    ramp(torch, lambda: burst(50), 20.0 if a.prewarm_ms > 0 else 0.0)
     for i in range(a.warmup):
         step(i)
     torch.cuda.synchronize()
